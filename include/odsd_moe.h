@@ -1,0 +1,156 @@
+/*
+ * odsd_moe.h -- C ABI of the MI355X (gfx950) MoE-block library, libodsd_moe.so.
+ *
+ * One hot path: router logits -> softmax -> top-k (optional renormalisation) ->
+ * stable dispatch by expert -> grouped W4A16 (group-128 asymmetric, fp16 scale/zero)
+ * SwiGLU experts -> deterministic weighted combine (+ residual), plus the RMSNorm that
+ * precedes it in a decoder layer.
+ *
+ * Conventions
+ *  - every pointer is a DEVICE pointer unless stated otherwise; all tensors are dense
+ *    row-major; `stream` is a hipStream_t passed as void* (NULL = the null stream);
+ *  - every call is asynchronous on `stream`, performs no host synchronisation, allocates
+ *    and frees nothing, and keeps no pointer after it returns;
+ *  - every call returns an odsd_status (0 = ok); nothing aborts or throws across the ABI;
+ *  - T tokens, H hidden size, E experts, K experts per token, I expert intermediate size,
+ *    P = T*K (token, k) pairs; pair p = t*K + k;
+ *  - activation dtype codes: ODSD_DT_F32 (float) or ODSD_DT_BF16 (bfloat16 bit patterns).
+ *
+ * Reference interfaces each entry point stands in for (paths relative to the
+ * potatoZhx/on_device_sd tree):
+ *   odsd_router_topk   Qwen3MoEGate.forward                    demo/src/layers/moe_layer.py:25-60
+ *                      Qwen3ModelRunner.route_experts          demo/src/model/qwen3_runner.py:86-119
+ *                      GPUOperators.router                     demo/src/operators/gpu_operators.py:48-69
+ *   odsd_dispatch      mask / torch.where per expert           demo/src/model/qwen3_runner.py:303-314
+ *   odsd_experts_w4    expert_forward_with_weights             demo/src/layers/mlp.py:209-231
+ *                      _execute_moe_with_placement             demo/src/model/qwen3_runner.py:269-385
+ *                      ExpertOperator.expert_forward           demo/src/operators/base_operator.py:19-34
+ *   odsd_moe_forward   Qwen3MoELayerWithWeights.forward        demo/src/layers/moe_layer.py:193-254
+ *                      ModelRunner.forward_moe                 demo/src/core/model_runner.py:175-193
+ *   odsd_rmsnorm       RMSNorm.rms_forward                     demo/src/layers/layernorm.py:21-27
+ *   odsd_w4_quantize   quantize_tensor (form, per group)       pre_exp/expert_skip_prediction/quant.py:85-108
+ *   odsd_w4_pack       (no counterpart: the reference holds fp16/bf16 weights only;
+ *                       parameter_loader.py:424-539 is where a loader would call it)
+ */
+#ifndef ODSD_MOE_H
+#define ODSD_MOE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ODSD_VERSION 100
+
+typedef enum odsd_status {
+    ODSD_OK = 0,
+    ODSD_ERR_NULL = 1,        /* a required pointer is NULL                              */
+    ODSD_ERR_SHAPE = 2,       /* a size is non-positive or violates a divisibility rule  */
+    ODSD_ERR_UNSUPPORTED = 3, /* valid but outside what the kernels cover (E, K limits)  */
+    ODSD_ERR_ALIGN = 4,       /* a pointer is not 16-byte aligned                        */
+    ODSD_ERR_WORKSPACE = 5,   /* workspace smaller than the *_workspace_bytes() answer   */
+    ODSD_ERR_LAUNCH = 6,      /* the HIP runtime refused a launch                        */
+    ODSD_ERR_DTYPE = 7        /* unknown dtype code                                      */
+} odsd_status;
+
+enum { ODSD_DT_F32 = 0, ODSD_DT_BF16 = 1 };
+
+/* Shape of one MoE layer call.  Rules: H % 128 == 0, I % 128 == 0, 1 <= K <= E <= 512,
+ * K <= 64, T >= 0 (T == 0 is a no-op). */
+typedef struct odsd_moe_shape {
+    int32_t T, H, E, K, I;
+    int32_t renorm;     /* 0: weights = softmax over all E gathered at the top-k
+                           1: those weights divided by their sum (== softmax over the K
+                              selected logits, the demo engine's top-k -> softmax)        */
+    int32_t act_dtype;  /* dtype of x, gate weight, residual and out_act                 */
+    int32_t reserved;
+} odsd_moe_shape;
+
+/* Per-expert weight table: E rows of 4 device addresses (as uint64):
+ *   [0] packed gate_up codes   [1] gate_up (scale, zero) pairs
+ *   [2] packed down codes      [3] down (scale, zero) pairs
+ * in the layout odsd_w4_pack writes.  A row whose first entry is 0 marks an expert whose
+ * weights are not available: its pairs contribute nothing (qwen3_runner.py:330-333).
+ * Substitution (qwen3_runner.py:322-329) is a row that points at another expert's arrays. */
+#define ODSD_TABLE_COLS 4
+
+int         odsd_version(void);
+const char *odsd_status_string(int status);
+
+/* ---- W4 storage ------------------------------------------------------------------- */
+/* Canonical form of one [N, Kd] matrix (nn.Linear layout, Kd = input size, Kd % 128 == 0):
+ *   q     uint8  [N, Kd/2]    code(2j) low nibble, code(2j+1) high nibble of byte j
+ *   scale fp16   [N, Kd/128]  zero fp16 [N, Kd/128];  w ~= (code - zero) * scale          */
+int odsd_w4_quantize(const void *w, int32_t w_dtype, int64_t N, int64_t Kd,
+                     uint8_t *q, uint16_t *scale, uint16_t *zero, void *stream);
+
+/* Bytes of the streaming layout of an [N, Kd] matrix (N % 16 == 0). */
+size_t odsd_w4_packed_q_bytes(int64_t N, int64_t Kd);
+size_t odsd_w4_packed_sz_bytes(int64_t N, int64_t Kd);
+
+/* Canonical -> streaming layout.  Source 16-row block b goes to destination block
+ * b*block_stride + block_offset, so gate_proj (stride 2, offset 0) and up_proj (stride 2,
+ * offset 1) interleave into one [2I, H] gate_up matrix; down_proj uses (1, 0). */
+int odsd_w4_pack(const uint8_t *q, const uint16_t *scale, const uint16_t *zero,
+                 int64_t N, int64_t Kd, int32_t block_stride, int32_t block_offset,
+                 uint32_t *qp, uint16_t *sz, void *stream);
+
+/* ---- RMSNorm ------------------------------------------------------------------------ */
+/* out = cast(x * rsqrt(mean(x^2) + eps)) * weight, cast BEFORE the weight multiply. */
+int odsd_rmsnorm(const void *x, const void *weight, int32_t dtype, int32_t T, int32_t H,
+                 float eps, void *out, void *stream);
+
+/* ---- Router ------------------------------------------------------------------------- */
+size_t odsd_router_workspace_bytes(const odsd_moe_shape *s);
+/* x [T,H], gate_w [E,H] in act_dtype.  Logits are accumulated in fp64.
+ * out_idx  int32 [T,K] experts in descending logit order, ties to the lower index
+ * out_w    float [T,K]
+ * out_idx64 (optional) the same indices as int64, the dtype torch.topk returns
+ * x_f16    (optional) fp16 copy of x [T,H], the operand format of odsd_experts_w4 */
+int odsd_router_topk(const odsd_moe_shape *s, const void *x, const void *gate_w,
+                     int32_t *out_idx, float *out_w, int64_t *out_idx64, void *x_f16,
+                     void *workspace, size_t workspace_bytes, void *stream);
+
+/* act_dtype [n] -> fp16 [n] (saturating); for callers that route elsewhere. */
+int odsd_convert_act_f16(const void *x, int32_t dtype, int64_t n, void *x_f16, void *stream);
+
+/* ---- Dispatch ----------------------------------------------------------------------- */
+/* Stable counting sort of the P pairs by expert id.
+ * counts [E], offsets [E+1], perm [P] pair -> slot (-1 if the id is outside [0,E)),
+ * inv [P] slot -> pair, slot_token [P] slot -> token (= inv / K). */
+int odsd_dispatch(const odsd_moe_shape *s, const int32_t *idx, int32_t *counts,
+                  int32_t *offsets, int32_t *perm, int32_t *inv, int32_t *slot_token,
+                  void *stream);
+
+/* ---- Experts + combine -------------------------------------------------------------- */
+size_t odsd_experts_workspace_bytes(const odsd_moe_shape *s);
+/* Grouped W4 gate_up -> SiLU*mul -> down over the dispatched pairs, then
+ *   moe[t] = sum_k w[t,k] * y[perm[t*K+k]]   (fp32, k order, one rounding)
+ * out_f32 (optional) float [T,H]  = moe (+ residual if given)
+ * out_act (optional) act_dtype [T,H] = cast(residual + cast(moe)) as the reference rounds it
+ * residual (optional) act_dtype [T,H]. */
+int odsd_experts_w4(const odsd_moe_shape *s, const void *x_f16, const uint64_t *table,
+                    const int32_t *idx, const float *w, const int32_t *counts,
+                    const int32_t *offsets, const int32_t *perm, const int32_t *slot_token,
+                    const void *residual, float *out_f32, void *out_act,
+                    void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---- Whole block -------------------------------------------------------------------- */
+size_t odsd_moe_workspace_bytes(const odsd_moe_shape *s);
+/* router -> dispatch -> experts -> combine in one call, no host round trip.
+ * norm_weight (optional): apply RMSNorm(x) first (x is then the residual stream and is
+ * also used as `residual` when add_residual != 0).
+ * Routing outputs out_idx/out_w/out_counts/out_offsets/out_perm are optional. */
+int odsd_moe_forward(const odsd_moe_shape *s, const void *x, const void *norm_weight,
+                     float eps, const void *gate_w, const uint64_t *table,
+                     int32_t add_residual, float *out_f32, void *out_act,
+                     int32_t *out_idx, float *out_w, int32_t *out_counts,
+                     int32_t *out_offsets, int32_t *out_perm,
+                     void *workspace, size_t workspace_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ODSD_MOE_H */

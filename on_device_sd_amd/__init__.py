@@ -1,0 +1,16 @@
+"""MI355X-native MoE block (router -> top-k -> dispatch -> W4A16 SwiGLU experts -> combine).
+
+Host code is Python on PyTorch-ROCm; all computation runs in hand-written gfx950 kernels
+behind the C ABI of ``include/odsd_moe.h`` (``libodsd_moe.so`` next to this file).
+"""
+from .core import (AttentionOutput, ExpertID, ExpertPlacement, LayerOutput, MoEConfig,
+                   RoutingResult)
+from . import _lib, ops, workloads
+from .w4 import W4ExpertBank, W4ExpertParams, build_table
+from .runner import (MoEOnlyStack, W4MoERunner, expert_forward_with_weights, moe_layer_forward)
+
+__all__ = [
+    "AttentionOutput", "ExpertID", "ExpertPlacement", "LayerOutput", "MoEConfig", "RoutingResult",
+    "W4ExpertBank", "W4ExpertParams", "build_table", "MoEOnlyStack", "W4MoERunner",
+    "expert_forward_with_weights", "moe_layer_forward", "ops", "workloads",
+]

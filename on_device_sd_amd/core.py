@@ -1,0 +1,104 @@
+"""Data types the engine and the runner exchange around the MoE block.
+
+Same names, fields and meaning as the reference's ``demo/src/core/model_runner.py:14-67``
+(RoutingResult, ExpertPlacement, LayerOutput, AttentionOutput), ``demo/src/core/types.py:19-29``
+(ExpertID) and the MoE part of ``demo/src/core/model.py:26-129`` (MoEConfig), so that engine
+code written against the reference works unchanged on top of this runner.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Dict, Optional, Set
+
+import torch
+
+
+@dataclass
+class ExpertID:
+    """Unique identifier of an expert (types.py:19-29)."""
+    layer_idx: int
+    expert_idx: int
+
+    def __hash__(self):
+        return hash((self.layer_idx, self.expert_idx))
+
+    def __str__(self):
+        return f"L{self.layer_idx}_E{self.expert_idx}"
+
+
+@dataclass
+class RoutingResult:
+    """What route_experts returns (model_runner.py:14-27).
+
+    topk_indices [T, K] int64 in descending-score order, topk_scores [T, K] float32.
+    ``dispatch`` is an optional cache of the device-side dispatch arrays that
+    route_experts already produced; forward_moe recomputes them when it is absent
+    (for example on a hand-built RoutingResult).
+    """
+    layer_idx: int
+    topk_indices: torch.Tensor
+    topk_scores: torch.Tensor
+    activated_expert_ids: Set[ExpertID]
+    dispatch: Optional[Any] = field(default=None, repr=False, compare=False)
+
+    @property
+    def top_k(self) -> int:
+        return self.topk_indices.shape[-1]
+
+
+@dataclass
+class ExpertPlacement:
+    """The engine's decision where each expert runs (model_runner.py:30-43)."""
+    gpu_expert_params: Dict[int, Dict[str, Any]]
+    cpu_expert_params: Dict[int, Dict[str, Any]]
+    substitution_map: Dict[int, int] = field(default_factory=dict)
+    routing_result: Optional[RoutingResult] = None
+
+
+@dataclass
+class LayerOutput:
+    """model_runner.py:46-58; metadata keys gpu_expert_count / cpu_expert_count /
+    substituted_count as in qwen3_runner.py:252-256."""
+    hidden_states: torch.Tensor
+    metadata: Dict[str, Any] = field(default_factory=dict)
+
+
+@dataclass
+class AttentionOutput:
+    """model_runner.py:61-67."""
+    hidden_states: torch.Tensor
+    post_attn_normed: torch.Tensor
+    residual: torch.Tensor
+
+
+@dataclass
+class MoEConfig:
+    """MoE-relevant subset of the reference MoEConfig (model.py:26-63) plus the two
+    knobs this implementation adds: ``norm_topk_prob`` and the W4 group size."""
+    hidden_size: int = 2048
+    num_hidden_layers: int = 48
+    num_experts: int = 128
+    num_experts_per_token: int = 8
+    moe_intermediate_size: int = 768
+    rms_norm_eps: float = 1e-6
+    torch_dtype: str = "bfloat16"
+    model_type: str = "qwen3_moe"
+    # True  = weights renormalised over the selected experts (the demo engine's
+    #         top-k -> softmax, moe_layer.py:49-54, and HF norm_topk_prob=True)
+    # False = softmax over all experts, gathered (Mixtral CoreInfer, core_moe.py:133-145)
+    norm_topk_prob: bool = True
+    w4_group_size: int = 128
+
+    @property
+    def is_moe(self) -> bool:
+        return self.num_experts > 1
+
+    def get_dtype(self) -> torch.dtype:
+        return {"float16": torch.float16, "bfloat16": torch.bfloat16,
+                "float32": torch.float32}.get(self.torch_dtype, torch.float16)
+
+    def get_expert_weight_size_bytes(self) -> int:
+        """Bytes of one expert in W4 group-128 storage (codes + fp16 scale + fp16 zero):
+        the 4-bit counterpart of model.py:111-115."""
+        params = 3 * self.moe_intermediate_size * self.hidden_size
+        return params // 2 + (params // self.w4_group_size) * 4

@@ -1,0 +1,94 @@
+// Entry points that tie the stages together: version/status strings and the whole-block
+// call (RMSNorm -> router -> dispatch -> experts -> combine) that never returns to the host
+// between stages.  Stands in for Qwen3MoELayerWithWeights.forward
+// (demo/src/layers/moe_layer.py:193-254) and for route_experts + forward_moe called back to
+// back (demo/src/model/qwen3_runner.py:86-119, :212-226) when the engine needs no decision
+// in between.
+#include "common.h"
+
+extern "C" int odsd_version(void) { return ODSD_VERSION; }
+
+extern "C" const char *odsd_status_string(int status) {
+    switch (status) {
+        case ODSD_OK: return "ok";
+        case ODSD_ERR_NULL: return "a required pointer is NULL";
+        case ODSD_ERR_SHAPE: return "bad shape (non-positive size or divisibility rule violated)";
+        case ODSD_ERR_UNSUPPORTED: return "shape outside the supported range (E <= 512, K <= 64)";
+        case ODSD_ERR_ALIGN: return "pointer not 16-byte aligned";
+        case ODSD_ERR_WORKSPACE: return "workspace too small";
+        case ODSD_ERR_LAUNCH: return "HIP launch failed";
+        case ODSD_ERR_DTYPE: return "unknown dtype code";
+        default: return "unknown status";
+    }
+}
+
+struct MoeLayout {
+    size_t router, xn, x16, idx, w, counts, offsets, perm, inv, slot_token, experts, total;
+};
+
+static MoeLayout moe_layout(const odsd_moe_shape *s) {
+    MoeLayout l;
+    const size_t T = s->T > 0 ? s->T : 1, P = T * s->K;
+    const size_t act = s->act_dtype == ODSD_DT_F32 ? 4 : 2;
+    size_t o = 0;
+    auto take = [&](size_t bytes) { const size_t at = o; o += odsd_round_up(bytes, 256); return at; };
+    l.router = take(odsd_router_workspace_bytes(s));
+    l.xn = take(T * s->H * act);
+    l.x16 = take(T * s->H * 2);
+    l.idx = take(P * 4);
+    l.w = take(P * 4);
+    l.counts = take((size_t)s->E * 4);
+    l.offsets = take((size_t)(s->E + 1) * 4);
+    l.perm = take(P * 4);
+    l.inv = take(P * 4);
+    l.slot_token = take(P * 4);
+    l.experts = take(odsd_experts_workspace_bytes(s));
+    l.total = o;
+    return l;
+}
+
+extern "C" size_t odsd_moe_workspace_bytes(const odsd_moe_shape *s) {
+    if (!s) return 0;
+    if (odsd_router_workspace_bytes(s) == 0 || odsd_experts_workspace_bytes(s) == 0) return 0;
+    return moe_layout(s).total;
+}
+
+extern "C" int odsd_moe_forward(const odsd_moe_shape *s, const void *x, const void *norm_weight, float eps,
+                                const void *gate_w, const uint64_t *table, int32_t add_residual,
+                                float *out_f32, void *out_act, int32_t *out_idx, float *out_w,
+                                int32_t *out_counts, int32_t *out_offsets, int32_t *out_perm,
+                                void *workspace, size_t workspace_bytes, void *stream) {
+    if (!s) return ODSD_ERR_NULL;
+    const size_t need = odsd_moe_workspace_bytes(s);
+    if (need == 0) return ODSD_ERR_SHAPE;
+    if (s->T == 0) return ODSD_OK;
+    if (!x || !gate_w || !table || !workspace) return ODSD_ERR_NULL;
+    if (!odsd_aligned16(workspace)) return ODSD_ERR_ALIGN;
+    if (workspace_bytes < need) return ODSD_ERR_WORKSPACE;
+    hipStream_t st = (hipStream_t)stream;
+    const MoeLayout l = moe_layout(s);
+    char *ws = (char *)workspace;
+    int32_t *idx = out_idx ? out_idx : (int32_t *)(ws + l.idx);
+    float *w = out_w ? out_w : (float *)(ws + l.w);
+    int32_t *counts = out_counts ? out_counts : (int32_t *)(ws + l.counts);
+    int32_t *offsets = out_offsets ? out_offsets : (int32_t *)(ws + l.offsets);
+    int32_t *perm = out_perm ? out_perm : (int32_t *)(ws + l.perm);
+    int32_t *inv = (int32_t *)(ws + l.inv);
+    int32_t *slot_token = (int32_t *)(ws + l.slot_token);
+    void *x16 = ws + l.x16;
+
+    const void *xin = x;
+    if (norm_weight) {
+        const int rc = odsd_rmsnorm(x, norm_weight, s->act_dtype, s->T, s->H, eps, ws + l.xn, stream);
+        if (rc != ODSD_OK) return rc;
+        xin = ws + l.xn;
+    }
+    int rc = odsd_launch_router(s, xin, gate_w, idx, w, nullptr, x16, ws + l.router,
+                                l.xn - l.router, st);
+    if (rc != ODSD_OK) return rc;
+    rc = odsd_launch_dispatch(s, idx, counts, offsets, perm, inv, slot_token, st);
+    if (rc != ODSD_OK) return rc;
+    return odsd_launch_experts(s, x16, table, idx, w, counts, offsets, perm, slot_token,
+                               add_residual ? x : nullptr, out_f32, out_act, ws + l.experts,
+                               l.total - l.experts, st);
+}

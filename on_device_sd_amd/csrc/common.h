@@ -1,0 +1,102 @@
+// Shared device helpers for the gfx950 MoE kernels (64-wide wavefronts throughout).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/odsd_moe.h"
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef double double4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+
+#define ODSD_WAVE 64
+#define ODSD_GROUP 128     // quantisation group (columns of the reduction dimension)
+#define ODSD_FP16_MAX 65504.0f
+
+// ---- bf16 <-> f32 (bf16 is carried as its 16-bit pattern) ------------------------------
+__device__ __forceinline__ float bf16_to_f32(uint16_t b) {
+    return __uint_as_float(((uint32_t)b) << 16);
+}
+// round-to-nearest-even, NaN kept quiet
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+template <typename T> struct ActIO;
+template <> struct ActIO<float> {
+    static constexpr int dtype = ODSD_DT_F32;
+    __device__ static __forceinline__ float load(const float *p, size_t i) { return p[i]; }
+    __device__ static __forceinline__ void store(float *p, size_t i, float v) { p[i] = v; }
+    // value after a round trip through the activation dtype
+    __device__ static __forceinline__ float round(float v) { return v; }
+};
+template <> struct ActIO<uint16_t> {
+    static constexpr int dtype = ODSD_DT_BF16;
+    __device__ static __forceinline__ float load(const uint16_t *p, size_t i) { return bf16_to_f32(p[i]); }
+    __device__ static __forceinline__ void store(uint16_t *p, size_t i, float v) { p[i] = f32_to_bf16(v); }
+    __device__ static __forceinline__ float round(float v) { return bf16_to_f32(f32_to_bf16(v)); }
+};
+
+// saturating f32 -> fp16 (round to nearest even)
+__device__ __forceinline__ half_t f32_to_f16_sat(float v) {
+    v = fminf(fmaxf(v, -ODSD_FP16_MAX), ODSD_FP16_MAX);
+    return (half_t)v;
+}
+
+// ---- wavefront helpers -------------------------------------------------------------------
+__device__ __forceinline__ int lane_id() { return (int)(threadIdx.x & (ODSD_WAVE - 1)); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, ODSD_WAVE);
+    return v;
+}
+__device__ __forceinline__ double wave_sum(double v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, ODSD_WAVE);
+    return v;
+}
+__device__ __forceinline__ float wave_min(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o, ODSD_WAVE));
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, ODSD_WAVE));
+    return v;
+}
+// number of set bits of `mask` below this lane
+__device__ __forceinline__ int mask_rank(uint64_t mask) {
+    return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32),
+                                     __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
+}
+
+// ---- host-side launch plumbing shared by the entry points ----------------------------------
+#define ODSD_CHECK_LAUNCH()                                   \
+    do {                                                      \
+        if (hipGetLastError() != hipSuccess) return ODSD_ERR_LAUNCH; \
+    } while (0)
+
+static inline bool odsd_aligned16(const void *p) { return (((uintptr_t)p) & 15u) == 0; }
+static inline size_t odsd_round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+// kernels implemented in the other translation units (host launchers)
+int odsd_launch_router(const odsd_moe_shape *s, const void *x, const void *gate_w, int32_t *idx,
+                       float *w, int64_t *idx64, void *x16, void *ws, size_t ws_bytes,
+                       hipStream_t st);
+int odsd_launch_dispatch(const odsd_moe_shape *s, const int32_t *idx, int32_t *counts,
+                         int32_t *offsets, int32_t *perm, int32_t *inv, int32_t *slot_token,
+                         hipStream_t st);
+int odsd_launch_experts(const odsd_moe_shape *s, const void *x16, const uint64_t *table,
+                        const int32_t *idx, const float *w, const int32_t *counts,
+                        const int32_t *offsets, const int32_t *perm, const int32_t *slot_token,
+                        const void *residual, float *out_f32, void *out_act, void *ws,
+                        size_t ws_bytes, hipStream_t st);

@@ -1,0 +1,293 @@
+// Router: logits = x . Wg^T accumulated in fp64, then softmax / top-k per token.
+//
+// Two kernels.
+//  1. router_partial_kernel: a split-K [T,H]x[H,E] product on the fp64 matrix cores
+//     (v_mfma_f64_16x16x4_f64).  One wavefront owns a tile of 16 tokens x (16*NE) experts
+//     over one K slice and writes fp64 partial logits.  fp64 accumulation makes the logits
+//     the exact dot product to ~1e-16, so the top-k choice does not depend on the
+//     summation order -- which is what lets the expert indices be bit-exact against a CPU
+//     restatement.  The tile with expert group 0 also writes the fp16 copy of x that the
+//     expert kernels consume.
+//  2. router_topk_kernel: one wavefront per token sums the partials in a fixed order,
+//     selects the K largest logits (ties to the lower index) by K rounds of a wavefront
+//     arg-max and computes the weights in fp32.
+//
+// Replaces: Qwen3MoEGate.forward (demo/src/layers/moe_layer.py:41-58), the stateless form
+// (:210-216) and GPUOperators.router (demo/src/operators/gpu_operators.py:48-69).
+#include "common.h"
+
+#define ROUTER_MAX_NE 4    // expert tiles (of 16) per wavefront
+#define ROUTER_MAX_V 8     // logits per lane in the top-k kernel -> E <= 512
+
+template <typename XT> struct Row8;
+template <> struct Row8<uint16_t> {  // 8 bf16 = 16 bytes
+    __device__ static __forceinline__ void load(const uint16_t *p, float (&v)[8]) {
+        const uint4_t u = *(const uint4_t *)p;
+        const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = __uint_as_float(w[i] << 16);
+            v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+        }
+    }
+};
+template <> struct Row8<float> {
+    __device__ static __forceinline__ void load(const float *p, float (&v)[8]) {
+        const float4_t a = *(const float4_t *)p, b = *(const float4_t *)(p + 4);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+        v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    }
+};
+
+// unit = (token tile, expert group, k split); 4 units (wavefronts) per workgroup.
+template <typename XT, int NE>
+__global__ __launch_bounds__(256) void router_partial_kernel(const XT *__restrict__ x,
+                                                             const XT *__restrict__ wg,
+                                                             double *__restrict__ partial,
+                                                             half_t *__restrict__ x16, int T, int H,
+                                                             int E, int S, int EG, int n_units) {
+    const int unit = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (unit >= n_units) return;
+    const int lane = lane_id();
+    const int r = lane & 15, kg = lane >> 4;
+    const int s = unit % S;
+    const int eg = (unit / S) % EG;
+    const int tt = unit / (S * EG);
+    const int Hs = H / S;
+    const int k0 = s * Hs;
+    const int t = tt * 16 + r;
+    const bool t_ok = t < T;
+
+    // Which (row, column) of the 16x16 result each of this lane's 4 accumulators holds is
+    // read back from the matrix core itself: D = A.B with A[i][0]=i, B[0][j]=1 gives D=i,
+    // and A[i][0]=1, B[0][j]=j gives D=j.
+    int di[4], dj[4];
+    {
+        const double4_t z = {0.0, 0.0, 0.0, 0.0};
+        const double a_i = kg == 0 ? (double)r : 0.0, one = kg == 0 ? 1.0 : 0.0;
+        const double4_t pi = __builtin_amdgcn_mfma_f64_16x16x4f64(a_i, one, z, 0, 0, 0);
+        const double4_t pj = __builtin_amdgcn_mfma_f64_16x16x4f64(one, a_i, z, 0, 0, 0);
+        di[0] = (int)pi.x; di[1] = (int)pi.y; di[2] = (int)pi.z; di[3] = (int)pi.w;
+        dj[0] = (int)pj.x; dj[1] = (int)pj.y; dj[2] = (int)pj.z; dj[3] = (int)pj.w;
+    }
+
+    double4_t acc[NE];
+#pragma unroll
+    for (int i = 0; i < NE; ++i) acc[i] = double4_t{0.0, 0.0, 0.0, 0.0};
+
+    const XT *xrow = x + (size_t)(t_ok ? t : 0) * H;
+    const XT *wrow[NE];
+    bool e_ok[NE];
+#pragma unroll
+    for (int i = 0; i < NE; ++i) {
+        const int e = (eg * NE + i) * 16 + r;
+        e_ok[i] = e < E;
+        wrow[i] = wg + (size_t)(e_ok[i] ? e : 0) * H;
+    }
+
+    for (int c = 0; c < Hs; c += 32) {
+        const int h = k0 + c + kg * 8;
+        float xa[8];
+        Row8<XT>::load(xrow + h, xa);
+        if (!t_ok) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) xa[j] = 0.0f;
+        }
+        if (x16 != nullptr && eg == 0 && t_ok) {
+            half8_t o;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) o[j] = f32_to_f16_sat(xa[j]);
+            *(half8_t *)(x16 + (size_t)t * H + h) = o;
+        }
+        double xd[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) xd[j] = (double)xa[j];
+#pragma unroll
+        for (int i = 0; i < NE; ++i) {
+            float wa[8];
+            Row8<XT>::load(wrow[i] + h, wa);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const double wd = e_ok[i] ? (double)wa[j] : 0.0;
+                acc[i] = __builtin_amdgcn_mfma_f64_16x16x4f64(xd[j], wd, acc[i], 0, 0, 0);
+            }
+        }
+    }
+
+#pragma unroll
+    for (int i = 0; i < NE; ++i) {
+        const double v[4] = {acc[i].x, acc[i].y, acc[i].z, acc[i].w};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int tq = tt * 16 + di[q];
+            const int eq = (eg * NE + i) * 16 + dj[q];
+            if (tq < T && eq < E) partial[((size_t)s * T + tq) * E + eq] = v[q];
+        }
+    }
+}
+
+// total order on doubles as unsigned keys: larger value <=> larger key
+__device__ __forceinline__ uint64_t order_key(double v) {
+    if (v == 0.0) v = 0.0;   // -0 and +0 compare equal, so they must share a key
+    const uint64_t b = (uint64_t)__double_as_longlong(v);
+    return (b >> 63) ? ~b : (b | 0x8000000000000000ull);
+}
+
+__global__ __launch_bounds__(256) void router_topk_kernel(const double *__restrict__ partial, int T, int E,
+                                                          int K, int S, int renorm,
+                                                          int32_t *__restrict__ idx,
+                                                          float *__restrict__ w,
+                                                          int64_t *__restrict__ idx64) {
+    const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= T) return;
+    const int lane = lane_id();
+
+    double lg[ROUTER_MAX_V];
+    uint64_t key[ROUTER_MAX_V];
+    uint32_t taken = 0;   // bit v set: expert lane + 64 v already selected
+#pragma unroll
+    for (int v = 0; v < ROUTER_MAX_V; ++v) {
+        const int e = lane + 64 * v;
+        double a = 0.0;
+        if (e < E)
+            for (int s = 0; s < S; ++s) a += partial[((size_t)s * T + t) * E + e];
+        lg[v] = a;
+        key[v] = order_key(a);
+        if (e >= E) taken |= 1u << v;
+    }
+
+    int my_e = 0;          // lane k keeps the k-th winner
+    double my_l = 0.0;
+    double l_max = 0.0;
+    for (int k = 0; k < K; ++k) {
+        // best remaining candidate of this lane: largest key, then lowest expert
+        uint64_t bk = 0;
+        int be = 0x7fffffff;
+        double bl = 0.0;
+#pragma unroll
+        for (int v = 0; v < ROUTER_MAX_V; ++v) {
+            if (!((taken >> v) & 1u)) {
+                if (be == 0x7fffffff || key[v] > bk) {
+                    bk = key[v];
+                    be = lane + 64 * v;
+                    bl = lg[v];
+                }
+            }
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const uint64_t ok = __shfl_xor(bk, o, ODSD_WAVE);
+            const int oe = __shfl_xor(be, o, ODSD_WAVE);
+            const double ol = __shfl_xor(bl, o, ODSD_WAVE);
+            const bool better = (oe != 0x7fffffff) &&
+                                (be == 0x7fffffff || ok > bk || (ok == bk && oe < be));
+            if (better) { bk = ok; be = oe; bl = ol; }
+        }
+        // every lane now agrees on (be, bl)
+        if ((be & 63) == lane) taken |= 1u << (be >> 6);
+        if (lane == k) { my_e = be; my_l = bl; }
+        if (k == 0) l_max = bl;
+    }
+
+    // weights in fp32; differences are taken in fp64 before the cast
+    float num = 0.0f;
+    if (lane < K) num = expf((float)(my_l - l_max));
+    float den;
+    if (renorm) {
+        den = wave_sum(num);
+    } else {
+        float part = 0.0f;
+#pragma unroll
+        for (int v = 0; v < ROUTER_MAX_V; ++v)
+            if (lane + 64 * v < E) part += expf((float)(lg[v] - l_max));
+        den = wave_sum(part);
+    }
+    if (lane < K) {
+        const size_t o = (size_t)t * K + lane;
+        idx[o] = my_e;
+        w[o] = num / den;
+        if (idx64) idx64[o] = (int64_t)my_e;
+    }
+}
+
+// ---- host side -----------------------------------------------------------------------------
+struct RouterPlan {
+    int NE, EG, TT, S;
+    size_t partial_bytes;
+};
+
+static RouterPlan router_plan(const odsd_moe_shape *s) {
+    RouterPlan p;
+    const int ET = (s->E + 15) / 16;
+    p.NE = ET >= 4 ? 4 : (ET >= 2 ? 2 : 1);
+    p.EG = (ET + p.NE - 1) / p.NE;
+    p.TT = (s->T + 15) / 16;
+    // split K until there are ~2048 wavefront units or the slices get down to 64 columns
+    int S = 1;
+    const int maxS = s->H / 64;
+    while (S * 2 <= maxS && (s->H / (S * 2)) % 32 == 0 && s->H % (S * 2) == 0 &&
+           (long)p.TT * p.EG * S < 2048)
+        S *= 2;
+    p.S = S;
+    p.partial_bytes = odsd_round_up((size_t)S * (size_t)(s->T > 0 ? s->T : 1) * s->E * sizeof(double), 256);
+    return p;
+}
+
+static int router_check(const odsd_moe_shape *s) {
+    if (!s) return ODSD_ERR_NULL;
+    if (s->T < 0 || s->H <= 0 || s->E <= 0 || s->K <= 0) return ODSD_ERR_SHAPE;
+    if (s->H % 128) return ODSD_ERR_SHAPE;
+    if (s->K > s->E) return ODSD_ERR_SHAPE;
+    if (s->E > 64 * ROUTER_MAX_V || s->K > 64) return ODSD_ERR_UNSUPPORTED;
+    if (s->act_dtype != ODSD_DT_F32 && s->act_dtype != ODSD_DT_BF16) return ODSD_ERR_DTYPE;
+    return ODSD_OK;
+}
+
+extern "C" size_t odsd_router_workspace_bytes(const odsd_moe_shape *s) {
+    if (router_check(s) != ODSD_OK) return 0;
+    return router_plan(s).partial_bytes;
+}
+
+template <typename XT, int NE>
+static void launch_partial(const RouterPlan &p, const odsd_moe_shape *s, const void *x, const void *gw,
+                           double *partial, void *x16, hipStream_t st) {
+    const int n_units = p.TT * p.EG * p.S;
+    router_partial_kernel<XT, NE><<<(n_units + 3) / 4, 256, 0, st>>>(
+        (const XT *)x, (const XT *)gw, partial, (half_t *)x16, s->T, s->H, s->E, p.S, p.EG, n_units);
+}
+
+int odsd_launch_router(const odsd_moe_shape *s, const void *x, const void *gate_w, int32_t *idx, float *w,
+                       int64_t *idx64, void *x16, void *ws, size_t ws_bytes, hipStream_t st) {
+    const int rc = router_check(s);
+    if (rc != ODSD_OK) return rc;
+    if (s->T == 0) return ODSD_OK;
+    if (!x || !gate_w || !idx || !w || !ws) return ODSD_ERR_NULL;
+    if (!odsd_aligned16(x) || !odsd_aligned16(gate_w) || !odsd_aligned16(ws) ||
+        (x16 && !odsd_aligned16(x16)))
+        return ODSD_ERR_ALIGN;
+    const RouterPlan p = router_plan(s);
+    if (ws_bytes < p.partial_bytes) return ODSD_ERR_WORKSPACE;
+    double *partial = (double *)ws;
+    const bool bf = s->act_dtype == ODSD_DT_BF16;
+#define ROUTER_GO(NEV)                                                                   \
+    do {                                                                                 \
+        if (bf) launch_partial<uint16_t, NEV>(p, s, x, gate_w, partial, x16, st);        \
+        else launch_partial<float, NEV>(p, s, x, gate_w, partial, x16, st);              \
+    } while (0)
+    if (p.NE == 4) ROUTER_GO(4);
+    else if (p.NE == 2) ROUTER_GO(2);
+    else ROUTER_GO(1);
+#undef ROUTER_GO
+    ODSD_CHECK_LAUNCH();
+    router_topk_kernel<<<(s->T + 3) / 4, 256, 0, st>>>(partial, s->T, s->E, s->K, p.S, s->renorm, idx, w,
+                                                        idx64);
+    ODSD_CHECK_LAUNCH();
+    return ODSD_OK;
+}
+
+extern "C" int odsd_router_topk(const odsd_moe_shape *s, const void *x, const void *gate_w,
+                                int32_t *out_idx, float *out_w, int64_t *out_idx64, void *x_f16,
+                                void *workspace, size_t workspace_bytes, void *stream) {
+    return odsd_launch_router(s, x, gate_w, out_idx, out_w, out_idx64, x_f16, workspace, workspace_bytes,
+                              (hipStream_t)stream);
+}

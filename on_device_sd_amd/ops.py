@@ -1,0 +1,273 @@
+"""Functional wrappers: torch tensors in, C-ABI calls on the current HIP stream, tensors out.
+
+torch is used for device memory and the stream handle only; every computation below runs in
+the hand-written gfx950 kernels of libodsd_moe.so.  Nothing here falls back to torch ops.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import MoeShape
+
+
+def _dtype_code(dt: torch.dtype) -> int:
+    if dt == torch.float32:
+        return _lib.DT_F32
+    if dt == torch.bfloat16:
+        return _lib.DT_BF16
+    raise TypeError(f"activation dtype {dt} is not supported (float32 or bfloat16)")
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _require_cuda(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("the MoE path runs on the GPU only: got a CPU tensor "
+                               "(there is no CPU fallback)")
+
+
+def make_shape(T: int, H: int, E: int, K: int, I: int, renorm: bool, dtype: torch.dtype) -> MoeShape:
+    return MoeShape(T, H, E, K, I, 1 if renorm else 0, _dtype_code(dtype), 0)
+
+
+def _workspace(nbytes: int, device) -> torch.Tensor:
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+
+
+# ------------------------------------------------------------------------------------------
+# W4 storage
+# ------------------------------------------------------------------------------------------
+def w4_quantize(w: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """[N, Kd] float32/bfloat16 weight -> canonical (q uint8 [N,Kd/2], scale fp16 [N,Kd/128],
+    zero fp16 [N,Kd/128])."""
+    _require_cuda(w)
+    lib = _lib.load()
+    w = w.contiguous()
+    n, kd = w.shape
+    q = torch.empty(n, kd // 2, dtype=torch.uint8, device=w.device)
+    scale = torch.empty(n, kd // 128, dtype=torch.float16, device=w.device)
+    zero = torch.empty_like(scale)
+    _lib.check(lib.odsd_w4_quantize(w.data_ptr(), _dtype_code(w.dtype), n, kd, q.data_ptr(),
+                                    scale.data_ptr(), zero.data_ptr(), _stream()), "odsd_w4_quantize")
+    return q, scale, zero
+
+
+def w4_packed_bytes(n: int, kd: int) -> Tuple[int, int]:
+    lib = _lib.load()
+    qb, sb = lib.odsd_w4_packed_q_bytes(n, kd), lib.odsd_w4_packed_sz_bytes(n, kd)
+    if qb == 0 or sb == 0:
+        raise ValueError(f"[{n}, {kd}] cannot be packed: rows must be a multiple of 16 and "
+                         "columns a multiple of 128")
+    return qb, sb
+
+
+def w4_pack_into(q: torch.Tensor, scale: torch.Tensor, zero: torch.Tensor, qp: torch.Tensor,
+                 sz: torch.Tensor, block_stride: int = 1, block_offset: int = 0) -> None:
+    """Canonical -> streaming layout, written into the uint8 buffers ``qp`` / ``sz``."""
+    _require_cuda(q, scale, zero, qp, sz)
+    lib = _lib.load()
+    n, kb = q.shape
+    _lib.check(lib.odsd_w4_pack(q.contiguous().data_ptr(), scale.contiguous().data_ptr(),
+                                zero.contiguous().data_ptr(), n, kb * 2, block_stride, block_offset,
+                                qp.data_ptr(), sz.data_ptr(), _stream()), "odsd_w4_pack")
+
+
+# ------------------------------------------------------------------------------------------
+# RMSNorm / conversion
+# ------------------------------------------------------------------------------------------
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6) -> torch.Tensor:
+    _require_cuda(x, weight)
+    lib = _lib.load()
+    x2 = x.contiguous().view(-1, x.shape[-1])
+    out = torch.empty_like(x2)
+    _lib.check(lib.odsd_rmsnorm(x2.data_ptr(), weight.to(x.dtype).contiguous().data_ptr(),
+                                _dtype_code(x.dtype), x2.shape[0], x2.shape[1], eps, out.data_ptr(),
+                                _stream()), "odsd_rmsnorm")
+    return out.view(x.shape)
+
+
+def to_f16(x: torch.Tensor) -> torch.Tensor:
+    _require_cuda(x)
+    lib = _lib.load()
+    x = x.contiguous()
+    out = torch.empty(x.shape, dtype=torch.float16, device=x.device)
+    _lib.check(lib.odsd_convert_act_f16(x.data_ptr(), _dtype_code(x.dtype), x.numel(), out.data_ptr(),
+                                        _stream()), "odsd_convert_act_f16")
+    return out
+
+
+# ------------------------------------------------------------------------------------------
+# Router / dispatch
+# ------------------------------------------------------------------------------------------
+def router_topk(x: torch.Tensor, gate_weight: torch.Tensor, top_k: int, renorm: bool,
+                want_f16: bool = False, want_int64: bool = False):
+    """x [T,H], gate_weight [E,H] (same dtype) -> (idx int32 [T,K], w float32 [T,K],
+    idx64 or None, x_f16 or None)."""
+    _require_cuda(x, gate_weight)
+    lib = _lib.load()
+    if gate_weight.dtype != x.dtype:
+        gate_weight = gate_weight.to(x.dtype)
+    x = x.contiguous()
+    gate_weight = gate_weight.contiguous()
+    T, H = x.shape
+    E = gate_weight.shape[0]
+    shape = make_shape(T, H, E, top_k, 128, renorm, x.dtype)
+    idx = torch.empty(T, top_k, dtype=torch.int32, device=x.device)
+    w = torch.empty(T, top_k, dtype=torch.float32, device=x.device)
+    idx64 = torch.empty(T, top_k, dtype=torch.int64, device=x.device) if want_int64 else None
+    x16 = torch.empty(T, H, dtype=torch.float16, device=x.device) if want_f16 else None
+    nbytes = lib.odsd_router_workspace_bytes(C.byref(shape))
+    if nbytes == 0:
+        raise _lib.OdsdError(f"router: unsupported shape T={T} H={H} E={E} K={top_k}")
+    ws = _workspace(nbytes, x.device)
+    _lib.check(lib.odsd_router_topk(C.byref(shape), x.data_ptr(), gate_weight.data_ptr(), idx.data_ptr(),
+                                    w.data_ptr(), _ptr(idx64), _ptr(x16), ws.data_ptr(), ws.numel(),
+                                    _stream()), "odsd_router_topk")
+    return idx, w, idx64, x16
+
+
+@dataclass
+class Dispatch:
+    """Device-side result of the stable sort of the (token, k) pairs by expert."""
+    counts: torch.Tensor      # int32 [E]
+    offsets: torch.Tensor     # int32 [E+1]
+    perm: torch.Tensor        # int32 [P]  pair -> slot
+    inv: torch.Tensor         # int32 [P]  slot -> pair
+    slot_token: torch.Tensor  # int32 [P]  slot -> token
+
+
+def dispatch(idx: torch.Tensor, num_experts: int) -> Dispatch:
+    _require_cuda(idx)
+    lib = _lib.load()
+    if idx.dtype != torch.int32:
+        idx = idx.to(torch.int32)
+    idx = idx.contiguous()
+    T, K = idx.shape
+    dev = idx.device
+    shape = MoeShape(T, 128, num_experts, K, 128, 0, _lib.DT_F32, 0)
+    d = Dispatch(torch.empty(num_experts, dtype=torch.int32, device=dev),
+                 torch.empty(num_experts + 1, dtype=torch.int32, device=dev),
+                 torch.empty(T * K, dtype=torch.int32, device=dev),
+                 torch.empty(T * K, dtype=torch.int32, device=dev),
+                 torch.empty(T * K, dtype=torch.int32, device=dev))
+    if T == 0:
+        d.counts.zero_()
+        d.offsets.zero_()
+        return d
+    _lib.check(lib.odsd_dispatch(C.byref(shape), idx.data_ptr(), d.counts.data_ptr(), d.offsets.data_ptr(),
+                                 d.perm.data_ptr(), d.inv.data_ptr(), d.slot_token.data_ptr(), _stream()),
+               "odsd_dispatch")
+    return d
+
+
+# ------------------------------------------------------------------------------------------
+# Experts + combine, whole block
+# ------------------------------------------------------------------------------------------
+def experts_w4(x_f16: torch.Tensor, table: torch.Tensor, idx: torch.Tensor, w: torch.Tensor,
+               disp: Dispatch, inter: int, act_dtype: torch.dtype,
+               residual: Optional[torch.Tensor] = None, want_f32: bool = True,
+               want_act: bool = False):
+    """Grouped W4 SwiGLU over the dispatched pairs and the weighted combine.
+    Returns (out_f32 or None, out_act or None), both [T, H]."""
+    _require_cuda(x_f16, table, idx, w)
+    lib = _lib.load()
+    T, H = x_f16.shape
+    E = table.shape[0]
+    K = idx.shape[1]
+    if idx.dtype != torch.int32:
+        idx = idx.to(torch.int32)
+    shape = make_shape(T, H, E, K, inter, False, act_dtype)
+    dev = x_f16.device
+    out32 = torch.empty(T, H, dtype=torch.float32, device=dev) if want_f32 else None
+    outa = torch.empty(T, H, dtype=act_dtype, device=dev) if want_act else None
+    if T == 0:
+        return out32, outa
+    nbytes = lib.odsd_experts_workspace_bytes(C.byref(shape))
+    if nbytes == 0:
+        raise _lib.OdsdError(f"experts: unsupported shape T={T} H={H} E={E} K={K} I={inter}")
+    ws = _workspace(nbytes, dev)
+    if residual is not None:
+        residual = residual.contiguous()
+        if residual.dtype != act_dtype:
+            raise TypeError("residual must have the activation dtype")
+    _lib.check(lib.odsd_experts_w4(C.byref(shape), x_f16.contiguous().data_ptr(), table.data_ptr(),
+                                   idx.contiguous().data_ptr(), w.contiguous().data_ptr(),
+                                   disp.counts.data_ptr(), disp.offsets.data_ptr(), disp.perm.data_ptr(),
+                                   disp.slot_token.data_ptr(), _ptr(residual), _ptr(out32), _ptr(outa),
+                                   ws.data_ptr(), ws.numel(), _stream()), "odsd_experts_w4")
+    return out32, outa
+
+
+@dataclass
+class MoeOutputs:
+    out_f32: Optional[torch.Tensor]
+    out_act: Optional[torch.Tensor]
+    idx: Optional[torch.Tensor]
+    w: Optional[torch.Tensor]
+    counts: Optional[torch.Tensor]
+    offsets: Optional[torch.Tensor]
+    perm: Optional[torch.Tensor]
+
+
+class MoeForwardPlan:
+    """Pre-sized buffers for repeated whole-block calls of one shape (no allocation per call)."""
+
+    def __init__(self, T: int, H: int, E: int, K: int, I: int, renorm: bool, dtype: torch.dtype,
+                 device, want_f32: bool = True, want_act: bool = True, want_routing: bool = True):
+        lib = _lib.load()
+        self.shape = make_shape(T, H, E, K, I, renorm, dtype)
+        nbytes = lib.odsd_moe_workspace_bytes(C.byref(self.shape))
+        if nbytes == 0:
+            raise _lib.OdsdError(f"moe_forward: unsupported shape T={T} H={H} E={E} K={K} I={I}")
+        self.ws = _workspace(nbytes, device)
+        self.out_f32 = torch.empty(T, H, dtype=torch.float32, device=device) if want_f32 else None
+        self.out_act = torch.empty(T, H, dtype=dtype, device=device) if want_act else None
+        P = T * K
+        if want_routing:
+            self.idx = torch.empty(T, K, dtype=torch.int32, device=device)
+            self.w = torch.empty(T, K, dtype=torch.float32, device=device)
+            self.counts = torch.empty(E, dtype=torch.int32, device=device)
+            self.offsets = torch.empty(E + 1, dtype=torch.int32, device=device)
+            self.perm = torch.empty(P, dtype=torch.int32, device=device)
+        else:
+            self.idx = self.w = self.counts = self.offsets = self.perm = None
+
+    def run(self, x: torch.Tensor, gate_weight: torch.Tensor, table: torch.Tensor,
+            norm_weight: Optional[torch.Tensor] = None, eps: float = 1e-6,
+            add_residual: bool = False, out_act: Optional[torch.Tensor] = None) -> MoeOutputs:
+        lib = _lib.load()
+        oa = out_act if out_act is not None else self.out_act
+        _lib.check(lib.odsd_moe_forward(
+            C.byref(self.shape), x.data_ptr(), _ptr(norm_weight), eps, gate_weight.data_ptr(),
+            table.data_ptr(), 1 if add_residual else 0, _ptr(self.out_f32), _ptr(oa), _ptr(self.idx),
+            _ptr(self.w), _ptr(self.counts), _ptr(self.offsets), _ptr(self.perm), self.ws.data_ptr(),
+            self.ws.numel(), _stream()), "odsd_moe_forward")
+        return MoeOutputs(self.out_f32, oa, self.idx, self.w, self.counts, self.offsets, self.perm)
+
+
+def moe_forward(x: torch.Tensor, gate_weight: torch.Tensor, table: torch.Tensor, top_k: int,
+                inter: int, renorm: bool, norm_weight: Optional[torch.Tensor] = None,
+                eps: float = 1e-6, add_residual: bool = False, want_f32: bool = True,
+                want_act: bool = True) -> MoeOutputs:
+    """One whole MoE block on a flat [T, H] input (allocating convenience form)."""
+    _require_cuda(x, gate_weight, table)
+    x = x.contiguous()
+    gate_weight = gate_weight.to(x.dtype).contiguous()
+    if norm_weight is not None:
+        norm_weight = norm_weight.to(x.dtype).contiguous()
+    T, H = x.shape
+    plan = MoeForwardPlan(T, H, gate_weight.shape[0], top_k, inter, renorm, x.dtype, x.device,
+                          want_f32, want_act)
+    return plan.run(x, gate_weight, table, norm_weight, eps, add_residual)

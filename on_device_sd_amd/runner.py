@@ -1,0 +1,220 @@
+"""Drop-in MoE part of the reference ModelRunner, on W4 experts resident in HBM.
+
+``W4MoERunner`` implements the two MoE methods of ``ModelRunner``
+(``demo/src/core/model_runner.py:149-193``) with the signatures and result types of
+``Qwen3ModelRunner`` (``demo/src/model/qwen3_runner.py:86-119, :212-226``):
+
+    route_experts(layer_idx, hidden_states) -> RoutingResult
+    forward_moe(layer_idx, attn_output, expert_placement) -> Tensor
+
+plus the stateless layer forms of ``demo/src/layers/moe_layer.py:93-107, :193-206`` and the
+functional expert of ``demo/src/layers/mlp.py:209-214``.  Attention, embedding and logits
+are not part of this path.
+
+Behaviour kept from the reference: 2-D or 3-D hidden states; ``routing_result is None`` gives
+a zero MoE contribution; experts missing from the placement are skipped; a substitution
+map uses the substitute's weights with the original expert's tokens and routing weights;
+``activated_expert_ids`` equals the set of unique selected experts.
+Deliberate differences: scores are float32 (the reference returns the model dtype); the
+combine is one fp32 gather-sum per token with a single rounding (the reference does one
+read-modify-write in the activation dtype per expert); an expert id repeated inside one
+token's top-k list contributes once per occurrence (the reference's indexed "+=" keeps one
+of them); experts placed on the CPU are refused, because every expert lives in HBM here.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from . import ops
+from .core import (AttentionOutput, ExpertID, ExpertPlacement, LayerOutput, MoEConfig,
+                   RoutingResult)
+from .w4 import W4ExpertBank, W4ExpertParams, build_table
+
+
+class W4MoERunner:
+    def __init__(self, config: MoEConfig, gate_weights: List[torch.Tensor],
+                 banks: List[W4ExpertBank], norm_weights: Optional[List[torch.Tensor]] = None):
+        """gate_weights[l]: [E, H] router weight of layer l (model dtype);
+        banks[l]: the layer's W4 experts; norm_weights[l]: post-attention RMSNorm weight."""
+        self.config = config
+        self.dtype = config.get_dtype()
+        self.device = banks[0].device
+        self.gate_weights = [g.to(device=self.device, dtype=self.dtype).contiguous() for g in gate_weights]
+        self.banks = banks
+        self.norm_weights = None if norm_weights is None else [
+            n.to(device=self.device, dtype=self.dtype).contiguous() for n in norm_weights]
+        self._table_cache: Dict[tuple, torch.Tensor] = {}
+
+    # -- ModelRunner interface -----------------------------------------------------------------
+    def get_config(self) -> MoEConfig:
+        return self.config
+
+    def get_num_layers(self) -> int:
+        return len(self.banks)
+
+    def route_experts(self, layer_idx: int, hidden_states: torch.Tensor) -> RoutingResult:
+        cfg = self.config
+        flat = hidden_states.reshape(-1, hidden_states.shape[-1])
+        idx32, w, idx64, _ = ops.router_topk(flat, self.gate_weights[layer_idx],
+                                             cfg.num_experts_per_token, cfg.norm_topk_prob,
+                                             want_int64=True)
+        disp = ops.dispatch(idx32, cfg.num_experts)
+        # the engine reads the activated set on the host between routing and execution
+        # (qwen3_runner.py:110-112): one small device-to-host copy of the E counts
+        counts = disp.counts.cpu().tolist()
+        activated = {ExpertID(layer_idx, e) for e, c in enumerate(counts) if c > 0}
+        return RoutingResult(layer_idx=layer_idx, topk_indices=idx64, topk_scores=w,
+                             activated_expert_ids=activated, dispatch=disp)
+
+    def forward_moe(self, layer_idx: int, attn_output: AttentionOutput,
+                    expert_placement: ExpertPlacement) -> torch.Tensor:
+        moe = self._execute_moe_with_placement(attn_output.post_attn_normed, expert_placement,
+                                               residual=attn_output.residual)
+        return moe
+
+    def forward_layer(self, layer_idx: int, hidden_states: torch.Tensor,
+                      expert_placement: Optional[ExpertPlacement] = None) -> LayerOutput:
+        """MoE-only layer: residual = h; h = RMSNorm(h); h = MoE(h); h = residual + h
+        (decoder_layer.py:126-140 without attention), through the separate
+        route_experts / forward_moe calls the engine loops use."""
+        if self.norm_weights is None:
+            raise RuntimeError("forward_layer needs the post-attention RMSNorm weights")
+        normed = ops.rmsnorm(hidden_states, self.norm_weights[layer_idx], self.config.rms_norm_eps)
+        routing = self.route_experts(layer_idx, normed)
+        if expert_placement is None:
+            expert_placement = ExpertPlacement(gpu_expert_params=self.banks[layer_idx].all_expert_params(),
+                                               cpu_expert_params={})
+        expert_placement.routing_result = routing
+        attn = AttentionOutput(hidden_states=hidden_states, post_attn_normed=normed,
+                               residual=hidden_states)
+        out = self.forward_moe(layer_idx, attn, expert_placement)
+        meta = {"gpu_expert_count": len(expert_placement.gpu_expert_params),
+                "cpu_expert_count": len(expert_placement.cpu_expert_params),
+                "substituted_count": len(expert_placement.substitution_map)}
+        return LayerOutput(hidden_states=out, metadata=meta)
+
+    # -- internals -----------------------------------------------------------------------------
+    def _placement_table(self, placement: ExpertPlacement) -> torch.Tensor:
+        params: Dict[int, W4ExpertParams] = {}
+        for src in (placement.gpu_expert_params, placement.cpu_expert_params):
+            for e, p in src.items():
+                if not isinstance(p, W4ExpertParams):
+                    raise TypeError(
+                        f"expert {e}: parameters are not W4 bundles resident in HBM; this runner "
+                        "executes every expert on the GPU and has no CPU expert path")
+                params[e] = p
+        key = (tuple(sorted((e, p.ptrs) for e, p in params.items())),
+               tuple(sorted(placement.substitution_map.items())))
+        tab = self._table_cache.get(key)
+        if tab is None:
+            if len(self._table_cache) > 64:
+                self._table_cache.clear()
+            tab = build_table(self.config.num_experts, params, placement.substitution_map, self.device)
+            self._table_cache[key] = tab
+        return tab
+
+    def _execute_moe_with_placement(self, hidden_states: torch.Tensor, placement: ExpertPlacement,
+                                    residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """qwen3_runner.py:269-385 (+ the residual add of :226 when ``residual`` is given)."""
+        routing = placement.routing_result
+        if routing is None:
+            return residual.clone() if residual is not None else torch.zeros_like(hidden_states)
+        shape = hidden_states.shape
+        flat = hidden_states.reshape(-1, shape[-1])
+        res = None if residual is None else residual.reshape(-1, shape[-1])
+        idx = routing.topk_indices.reshape(flat.shape[0], -1)
+        disp = routing.dispatch
+        if disp is None:
+            idx = idx.to(device=flat.device, dtype=torch.int32)
+            disp = ops.dispatch(idx, self.config.num_experts)
+        scores = routing.topk_scores.reshape(flat.shape[0], -1).to(device=flat.device,
+                                                                  dtype=torch.float32)
+        table = self._placement_table(placement)
+        _, out = ops.experts_w4(ops.to_f16(flat), table, idx, scores, disp,
+                                self.config.moe_intermediate_size, flat.dtype, residual=res,
+                                want_f32=False, want_act=True)
+        return out.view(shape)
+
+
+# -- stateless forms ---------------------------------------------------------------------------
+def moe_layer_forward(hidden_states: torch.Tensor, gate_weight: torch.Tensor,
+                      expert_weights_dict: Dict[int, W4ExpertParams], num_experts: int,
+                      num_experts_per_token: int, moe_intermediate_size: int,
+                      norm_topk_prob: bool = True, return_f32: bool = False) -> torch.Tensor:
+    """Qwen3MoELayerWithWeights.forward (moe_layer.py:193-254): [B,S,H] or [T,H] in, same shape
+    out, no residual.  ``expert_weights_dict`` maps expert id -> W4 bundle; ids that are not
+    in it are skipped."""
+    shape = hidden_states.shape
+    flat = hidden_states.reshape(-1, shape[-1])
+    table = build_table(num_experts, expert_weights_dict, None, flat.device)
+    o = ops.moe_forward(flat, gate_weight, table, num_experts_per_token, moe_intermediate_size,
+                        norm_topk_prob, want_f32=return_f32, want_act=not return_f32)
+    return (o.out_f32 if return_f32 else o.out_act).view(shape)
+
+
+def expert_forward_with_weights(x: torch.Tensor, params: W4ExpertParams,
+                                return_f32: bool = False) -> torch.Tensor:
+    """mlp.py:209-231 for one W4 expert: down(silu(gate(x)) * up(x)) on every row of x."""
+    shape = x.shape
+    flat = x.reshape(-1, shape[-1])
+    T = flat.shape[0]
+    dev = flat.device
+    idx = torch.zeros(T, 1, dtype=torch.int32, device=dev)
+    w = torch.ones(T, 1, dtype=torch.float32, device=dev)
+    table = torch.tensor([params.ptrs], dtype=torch.int64).to(dev)
+    disp = ops.dispatch(idx, 1)
+    o32, oa = ops.experts_w4(ops.to_f16(flat), table, idx, w, disp, params.bank.inter, flat.dtype,
+                             want_f32=return_f32, want_act=not return_f32)
+    return (o32 if return_f32 else oa).view(shape)
+
+
+class MoEOnlyStack:
+    """L layers of RMSNorm -> MoE -> residual on a flat [T,H] hidden state, each layer one
+    whole-block call with no host round trip; the hidden state ping-pongs between two
+    buffers.  ``capture()`` records the L calls into a HIP graph for launch-bound shapes."""
+
+    def __init__(self, config: MoEConfig, gate_weights: List[torch.Tensor],
+                 norm_weights: List[torch.Tensor], banks: List[W4ExpertBank], T: int):
+        self.config = config
+        self.dtype = config.get_dtype()
+        self.device = banks[0].device
+        self.L = len(banks)
+        self.gate = [g.to(device=self.device, dtype=self.dtype).contiguous() for g in gate_weights]
+        self.norm = [n.to(device=self.device, dtype=self.dtype).contiguous() for n in norm_weights]
+        self.tables = [b.table() for b in banks]
+        self.banks = banks
+        self.T = T
+        self.plan = ops.MoeForwardPlan(T, config.hidden_size, config.num_experts,
+                                       config.num_experts_per_token, config.moe_intermediate_size,
+                                       config.norm_topk_prob, self.dtype, self.device,
+                                       want_f32=False, want_act=False, want_routing=False)
+        self.buf = [torch.empty(T, config.hidden_size, dtype=self.dtype, device=self.device)
+                    for _ in range(2)]
+        self.graph = None
+
+    def _run_layers(self):
+        for l in range(self.L):
+            self.plan.run(self.buf[l & 1], self.gate[l], self.tables[l], self.norm[l],
+                          self.config.rms_norm_eps, add_residual=True, out_act=self.buf[(l + 1) & 1])
+
+    def capture(self):
+        """Record the stack into a HIP graph (all kernels, no memset nodes)."""
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            self._run_layers()   # warm-up outside capture
+        torch.cuda.current_stream().wait_stream(s)
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            self._run_layers()
+        self.graph = g
+
+    def forward(self, hidden: torch.Tensor) -> torch.Tensor:
+        self.buf[0].copy_(hidden)
+        if self.graph is not None:
+            self.graph.replay()
+        else:
+            self._run_layers()
+        return self.buf[self.L & 1]

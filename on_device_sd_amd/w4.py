@@ -1,0 +1,128 @@
+"""HBM-resident W4 expert storage.
+
+One ``W4ExpertBank`` per MoE layer keeps all experts of the layer in four stacked device
+allocations (packed gate_up codes, gate_up (scale, zero), packed down codes, down
+(scale, zero)) in the streaming layout the kernels read, and hands out per-expert parameter
+dicts with the keys the reference loader uses ('gate_proj', 'up_proj', 'down_proj';
+``demo/src/memory/parameter_loader.py:480-491``).  The engine only passes those dicts
+through (``demo/src/execution/model_runner_utils.py:62-79``); the runner turns them into the
+device pointer table the kernels index by expert id.
+"""
+from __future__ import annotations
+
+from typing import Dict, Iterable, Optional, Tuple
+
+import torch
+
+from . import ops
+
+
+class W4Proj:
+    """Handle of one projection of one expert inside a bank (what the dict values are).
+    It mimics the few tensor attributes engine code looks at."""
+
+    def __init__(self, bank: "W4ExpertBank", expert: int, name: str, shape: Tuple[int, int]):
+        self.bank, self.expert, self.name, self.shape = bank, expert, name, shape
+
+    @property
+    def device(self):
+        return self.bank.device
+
+    @property
+    def dtype(self):
+        return torch.uint8
+
+    def __repr__(self):
+        return f"W4Proj({self.name}, expert={self.expert}, shape={self.shape})"
+
+
+class W4ExpertParams(dict):
+    """{'gate_proj', 'up_proj', 'down_proj'} -> W4Proj, plus the four device addresses."""
+
+    def __init__(self, bank: "W4ExpertBank", expert: int):
+        H, I = bank.hidden, bank.inter
+        super().__init__(gate_proj=W4Proj(bank, expert, "gate_proj", (I, H)),
+                         up_proj=W4Proj(bank, expert, "up_proj", (I, H)),
+                         down_proj=W4Proj(bank, expert, "down_proj", (H, I)))
+        self.bank = bank
+        self.expert = expert
+
+    @property
+    def ptrs(self) -> Tuple[int, int, int, int]:
+        return self.bank.expert_ptrs(self.expert)
+
+
+class W4ExpertBank:
+    def __init__(self, num_experts: int, hidden: int, inter: int, device="cuda"):
+        if hidden % 128 or inter % 128:
+            raise ValueError("hidden and intermediate sizes must be multiples of 128")
+        self.num_experts, self.hidden, self.inter = num_experts, hidden, inter
+        self.device = torch.device(device)
+        self.gu_q_bytes, self.gu_sz_bytes = ops.w4_packed_bytes(2 * inter, hidden)
+        self.dn_q_bytes, self.dn_sz_bytes = ops.w4_packed_bytes(hidden, inter)
+        E = num_experts
+        mk = lambda n: torch.zeros(E, n, dtype=torch.uint8, device=self.device)
+        self.gu_q, self.gu_sz = mk(self.gu_q_bytes), mk(self.gu_sz_bytes)
+        self.dn_q, self.dn_sz = mk(self.dn_q_bytes), mk(self.dn_sz_bytes)
+        self.loaded = [False] * E
+        self._table: Optional[torch.Tensor] = None
+
+    # -- sizes -------------------------------------------------------------------------------
+    @property
+    def bytes_per_expert(self) -> int:
+        return self.gu_q_bytes + self.gu_sz_bytes + self.dn_q_bytes + self.dn_sz_bytes
+
+    # -- loading -----------------------------------------------------------------------------
+    def load_canonical(self, e: int, gate, up, down) -> None:
+        """gate/up/down: canonical (q, scale, zero) triples on the device."""
+        ops.w4_pack_into(*gate, self.gu_q[e], self.gu_sz[e], 2, 0)
+        ops.w4_pack_into(*up, self.gu_q[e], self.gu_sz[e], 2, 1)
+        ops.w4_pack_into(*down, self.dn_q[e], self.dn_sz[e], 1, 0)
+        self.loaded[e] = True
+        self._table = None
+
+    def load_expert(self, e: int, gate_w: torch.Tensor, up_w: torch.Tensor, down_w: torch.Tensor,
+                    keep_canonical: bool = False):
+        """Quantise one expert's [I,H], [I,H], [H,I] weights on the device and pack them."""
+        canon = tuple(ops.w4_quantize(w.to(self.device)) for w in (gate_w, up_w, down_w))
+        self.load_canonical(e, *canon)
+        return canon if keep_canonical else None
+
+    # -- views -------------------------------------------------------------------------------
+    def expert_ptrs(self, e: int) -> Tuple[int, int, int, int]:
+        return (self.gu_q[e].data_ptr(), self.gu_sz[e].data_ptr(),
+                self.dn_q[e].data_ptr(), self.dn_sz[e].data_ptr())
+
+    def expert_params(self, e: int) -> W4ExpertParams:
+        if not self.loaded[e]:
+            raise KeyError(f"expert {e} has not been loaded")
+        return W4ExpertParams(self, e)
+
+    def all_expert_params(self) -> Dict[int, W4ExpertParams]:
+        return {e: self.expert_params(e) for e in range(self.num_experts) if self.loaded[e]}
+
+    def table(self) -> torch.Tensor:
+        """int64 [E, 4] device pointer table with every loaded expert present."""
+        if self._table is None:
+            rows = [self.expert_ptrs(e) if self.loaded[e] else (0, 0, 0, 0)
+                    for e in range(self.num_experts)]
+            self._table = torch.tensor(rows, dtype=torch.int64).to(self.device)
+        return self._table
+
+
+def build_table(num_experts: int, params: Dict[int, W4ExpertParams],
+                substitution: Optional[Dict[int, int]] = None, device="cuda") -> torch.Tensor:
+    """Pointer table for an arbitrary placement: row e points at params[e], or at
+    params[substitution[e]], or is 0 (expert skipped)."""
+    substitution = substitution or {}
+    rows = []
+    for e in range(num_experts):
+        src = e if e in params else substitution.get(e)
+        if src is not None and src in params:
+            p = params[src]
+            if not isinstance(p, W4ExpertParams):
+                raise TypeError(f"expert {src}: parameters are not W4 bundles of a W4ExpertBank")
+            rows.append(p.ptrs)
+        else:
+            rows.append((0, 0, 0, 0))
+    return torch.tensor(rows, dtype=torch.int64).to(device)

@@ -1,0 +1,182 @@
+"""Stage-by-stage parity of the HIP path (through the C ABI) against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_oracle as orc
+from tests.helpers import canon_to_oracle, check_output
+
+pytestmark = pytest.mark.gpu
+
+
+def _ops():
+    from on_device_sd_amd import ops
+    return ops
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(64, 512), (48, 1024), (16, 128)])
+def test_quantize_bit_exact(dev, dtype, shape):
+    print("quantize", dtype, shape, flush=True)
+    g = torch.Generator().manual_seed(1)
+    w = (torch.randn(*shape, generator=g) * 0.02).to(dtype)
+    w[3, :128] = 0.25            # constant group: scale guard
+    w[5, 128:256] = w[5, 128:256].abs() + 0.5   # all-positive group: negative zero point
+    q, s, z = _ops().w4_quantize(w.to(dev))
+    qo, so, zo = orc.quantize_w4(w.float().numpy())
+    assert np.array_equal(s.cpu().numpy().view(np.uint16), so.view(np.uint16))
+    assert np.array_equal(z.cpu().numpy().view(np.uint16), zo.view(np.uint16))
+    assert np.array_equal(q.cpu().numpy(), qo)
+
+
+@pytest.mark.parametrize("stride,offset", [(1, 0), (2, 0), (2, 1)])
+def test_pack_bit_exact(dev, stride, offset):
+    print("pack", stride, offset, flush=True)
+    rng = np.random.default_rng(2)
+    n, kd = 64, 384
+    q = rng.integers(0, 256, size=(n, kd // 2), dtype=np.uint8)
+    s = rng.standard_normal((n, kd // 128)).astype(np.float16)
+    z = rng.standard_normal((n, kd // 128)).astype(np.float16)
+    ops = _ops()
+    nblk = n // 16 * stride
+    qp = torch.zeros(nblk * (kd // 128) * 64 * 16, dtype=torch.uint8, device=dev)
+    sz = torch.zeros(nblk * (kd // 128) * 16 * 4, dtype=torch.uint8, device=dev)
+    ops.w4_pack_into(torch.from_numpy(q).to(dev), torch.from_numpy(s).to(dev), torch.from_numpy(z).to(dev),
+                     qp, sz, stride, offset)
+    qpo, szo = orc.pack_w4(q, s, z, stride, offset)
+    assert np.array_equal(qp.cpu().numpy().view(np.uint32).reshape(qpo.shape), qpo)
+    assert np.array_equal(sz.cpu().numpy().view(np.uint16), szo.view(np.uint16).reshape(-1))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rmsnorm(dev, dtype):
+    print("rmsnorm", dtype, flush=True)
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn(37, 768, generator=g) * 3).to(dtype)
+    w = (1 + 0.1 * torch.randn(768, generator=g)).to(dtype)
+    got = _ops().rmsnorm(x.to(dev), w.to(dev), 1e-6).cpu()
+    ref = orc.rmsnorm(x, w, 1e-6)
+    if dtype == torch.bfloat16:
+        # bit-exact up to rare 1-ulp flips where the fp32 value sits on a rounding boundary
+        diff = (got.view(torch.int16).int() - ref.view(torch.int16).int()).abs()
+        assert diff.max().item() <= 1 and (diff > 0).float().mean().item() < 1e-3
+    else:
+        torch.testing.assert_close(got, ref, rtol=2e-7, atol=0)
+
+
+ROUTER_CASES = [
+    # T, H, E, K, renorm, dtype
+    (32, 512, 8, 2, False, torch.float32),
+    (5, 4096, 8, 2, False, torch.bfloat16),
+    (160, 4096, 8, 2, False, torch.bfloat16),
+    (64, 2048, 128, 8, True, torch.bfloat16),
+    (33, 256, 60, 6, True, torch.float32),      # ragged token tile, E not a multiple of 16
+    (1, 128, 4, 4, True, torch.bfloat16),       # K == E
+    (300, 1024, 256, 8, False, torch.bfloat16), # 4 logits per lane
+]
+
+
+@pytest.mark.parametrize("T,H,E,K,renorm,dtype", ROUTER_CASES)
+def test_router_indices_bit_exact(dev, T, H, E, K, renorm, dtype):
+    print("router", T, H, E, K, renorm, dtype, flush=True)
+    g = torch.Generator().manual_seed(T * 7 + E)
+    x = torch.randn(T, H, generator=g).to(dtype)
+    wg = (torch.randn(E, H, generator=g) * 0.02).to(dtype)
+    idx, w, idx64, x16 = _ops().router_topk(x.to(dev), wg.to(dev), K, renorm, want_f16=True, want_int64=True)
+    idx_o, w_o = orc.route(orc.router_logits(x, wg), K, renorm)
+    assert np.array_equal(idx.cpu().numpy(), idx_o)
+    assert np.array_equal(idx64.cpu().numpy(), idx_o.astype(np.int64))
+    np.testing.assert_allclose(w.cpu().numpy(), w_o, rtol=2e-6, atol=1e-7)
+    assert torch.equal(x16.cpu(), x.to(torch.float16))
+    if renorm:
+        np.testing.assert_allclose(w.cpu().numpy().sum(-1), 1.0, atol=1e-5)
+
+
+def test_router_ties_lower_index_first(dev):
+    print("router ties", flush=True)
+    # identical gate rows give exactly equal logits: ties must go to the lower expert id
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(7, 256, generator=g).to(torch.bfloat16)
+    row = (torch.randn(1, 256, generator=g) * 0.02).to(torch.bfloat16)
+    wg = row.repeat(16, 1)
+    idx, w, _, _ = _ops().router_topk(x.to(dev), wg.to(dev), 4, True)
+    assert np.array_equal(idx.cpu().numpy(), np.tile(np.arange(4, dtype=np.int32), (7, 1)))
+    np.testing.assert_allclose(w.cpu().numpy(), 0.25, rtol=1e-6)
+    # all-zero input: every logit is +-0, again a full tie
+    idx, _, _, _ = _ops().router_topk(torch.zeros(3, 256, dtype=torch.bfloat16, device=dev),
+                                      (torch.randn(16, 256, generator=g) * 0.02).to(torch.bfloat16).to(dev), 4, False)
+    assert np.array_equal(idx.cpu().numpy(), np.tile(np.arange(4, dtype=np.int32), (3, 1)))
+
+
+@pytest.mark.parametrize("T,K,E", [(32, 2, 8), (5, 2, 8), (160, 2, 8), (64, 8, 128), (256, 8, 128),
+                                   (4096, 8, 128), (1, 1, 1), (700, 3, 40)])
+def test_dispatch_bit_exact(dev, T, K, E):
+    print("dispatch", T, K, E, flush=True)
+    rng = np.random.default_rng(T + K + E)
+    # distinct experts per token, popularity skewed
+    p = 1.0 / (np.arange(E) + 1.0)
+    p /= p.sum()
+    idx = np.stack([rng.choice(E, size=K, replace=False, p=p) for _ in range(T)]).astype(np.int32)
+    d = _ops().dispatch(torch.from_numpy(idx).to(dev), E)
+    c, o, perm, inv = orc.dispatch(idx, E)
+    assert np.array_equal(d.counts.cpu().numpy(), c)
+    assert np.array_equal(d.offsets.cpu().numpy(), o)
+    assert np.array_equal(d.perm.cpu().numpy(), perm)
+    assert np.array_equal(d.inv.cpu().numpy(), inv)
+    assert np.array_equal(d.slot_token.cpu().numpy(), inv // K)
+
+
+def test_dispatch_duplicates_and_out_of_range(dev):
+    print("dispatch dup/oob", flush=True)
+    idx = np.array([[0, 0], [3, 9], [-1, 2], [2, 2]], dtype=np.int32)
+    d = _ops().dispatch(torch.from_numpy(idx).to(dev), 4)
+    c, o, perm, inv = orc.dispatch(idx, 4)
+    assert np.array_equal(d.counts.cpu().numpy(), c)
+    assert np.array_equal(d.offsets.cpu().numpy(), o)
+    assert np.array_equal(d.perm.cpu().numpy(), perm)
+    assert np.array_equal(d.inv.cpu().numpy(), inv)
+
+
+def _small_layer(dev, T, H, E, K, I, dtype, seed, renorm=True):
+    import on_device_sd_amd as odsd
+    g = torch.Generator().manual_seed(seed)
+    wg = (torch.randn(E, H, generator=g) * 0.02).to(dtype)
+    bank = odsd.W4ExpertBank(E, H, I, dev)
+    experts = {}
+    for e in range(E):
+        canon = bank.load_expert(e, torch.randn(I, H, generator=g) * 0.02, torch.randn(I, H, generator=g) * 0.02,
+                                 torch.randn(H, I, generator=g) * 0.02, keep_canonical=True)
+        experts[e] = canon_to_oracle(canon)
+    x = torch.randn(T, H, generator=g).to(dtype)
+    return wg, bank, experts, x
+
+
+EXPERT_CASES = [
+    # T, H, E, K, I, dtype
+    (32, 512, 8, 2, 1024, torch.float32),     # config 1 shape
+    (3, 256, 4, 2, 128, torch.bfloat16),      # fewer rows than one MFMA block
+    (70, 384, 4, 2, 640, torch.bfloat16),     # >16 rows per expert, ragged row blocks (I/16 = 40)
+    (200, 256, 2, 2, 256, torch.bfloat16),    # 200 rows per expert: several passes
+    (64, 2048, 128, 8, 768, torch.bfloat16),  # config 3 shape (uniform routing)
+]
+
+
+@pytest.mark.parametrize("T,H,E,K,I,dtype", EXPERT_CASES)
+def test_moe_forward_vs_oracle(dev, T, H, E, K, I, dtype):
+    print("moe_forward", T, H, E, K, I, dtype, flush=True)
+    ops = _ops()
+    wg, bank, experts, x = _small_layer(dev, T, H, E, K, I, dtype, seed=T + H)
+    out = ops.moe_forward(x.to(dev), wg.to(dev), bank.table(), K, I, renorm=True)
+    ref, idx, w = orc.moe_block(x, wg, experts, K, True)
+    assert np.array_equal(out.idx.cpu().numpy(), idx)
+    c, o, perm, _ = orc.dispatch(idx, E)
+    assert np.array_equal(out.counts.cpu().numpy(), c)
+    assert np.array_equal(out.offsets.cpu().numpy(), o)
+    assert np.array_equal(out.perm.cpu().numpy(), perm)
+    mx, mean = check_output(out.out_f32, ref)
+    print(f"  max-abs {mx:.3e} mean-abs {mean:.3e}", flush=True)
+    # the activation-dtype output is the fp32 one rounded once
+    assert torch.equal(out.out_act.cpu(), out.out_f32.cpu().to(dtype))
+    # determinism: a second run gives the same bits
+    out2 = ops.moe_forward(x.to(dev), wg.to(dev), bank.table(), K, I, renorm=True)
+    assert torch.equal(out2.out_f32, out.out_f32)
