@@ -43,6 +43,10 @@ SIGNATURES = {
     "odsd_dispatch": (C.c_int, [_SP, _P, _P, _P, _P, _P, _P, _P]),
     "odsd_experts_workspace_bytes": (C.c_size_t, [_SP]),
     "odsd_experts_w4": (C.c_int, [_SP, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, C.c_size_t, _P]),
+    "odsd_w4_gate_up_silu": (C.c_int, [_SP, _P, _P, _P, _P, _P, _P, _P]),
+    "odsd_w4_down_splits": (C.c_int32, [_SP]),
+    "odsd_w4_down": (C.c_int, [_SP, _P, _P, _P, _P, _P, _P]),
+    "odsd_combine": (C.c_int, [_SP, _P, _P, _P, _P, _P, _P, _P, _P, _P]),
     "odsd_moe_workspace_bytes": (C.c_size_t, [_SP]),
     "odsd_moe_forward": (C.c_int, [_SP, _P, _P, C.c_float, _P, _P, C.c_int32, _P, _P, _P, _P, _P, _P,
                                    _P, _P, C.c_size_t, _P]),

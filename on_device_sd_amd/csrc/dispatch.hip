@@ -78,6 +78,7 @@ int odsd_launch_dispatch(const odsd_moe_shape *s, const int32_t *idx, int32_t *c
     if (s->T < 0 || s->E <= 0 || s->K <= 0) return ODSD_ERR_SHAPE;
     if ((int64_t)s->T * s->K > 0x7fffffffLL) return ODSD_ERR_SHAPE;
     if (!idx || !counts || !offsets || !perm || !inv || !slot_token) return ODSD_ERR_NULL;
+    if (s->T == 0) return ODSD_OK;
     const int P = s->T * s->K;
     const int threads = P <= 4096 ? 256 : 1024;
     dispatch_kernel<<<s->E, threads, 0, st>>>(idx, P, s->K, s->E, counts, offsets, perm, inv, slot_token);

@@ -22,7 +22,10 @@
 // and the indexed "+=" combine (:363, :376).
 #include "common.h"
 
-#define XS_STRIDE 136   // halfs per LDS row: 128 + 8 (16-byte skew between rows)
+
+typedef __attribute__((address_space(1))) uint4_t global_u4;
+typedef __attribute__((address_space(1))) uint32_t global_u32;
+typedef __attribute__((address_space(1))) char global_char;
 
 struct GemmParams {
     const uint64_t *table;   // [E][4]
@@ -40,17 +43,33 @@ struct GemmParams {
     int gper;                // groups per split
     int ldo;                 // I (MODE 0) or H (MODE 1)
     int P;
+    int E;
     int n_wg;                // E * nchunks * KS
     int wg_per_xcd;          // ceil(n_wg / 8)
 };
 
 __device__ __forceinline__ half2_t as_half2(uint32_t u) { return __builtin_bit_cast(half2_t, u); }
 
+// Constants of the code -> fp16 bit trick.  (x & mask) | magic is one VOP3 instruction
+// (v_and_or_b32), but gfx9 VOP3 takes no literal and a single scalar operand, so with
+// compile-time constants the compiler emits v_and + v_or.  Passing the constants through an
+// empty asm once per kernel makes them opaque register values (masks in SGPRs, the magic
+// number in a VGPR), and the fused form is selected.
+struct DequantConsts {
+    uint32_t m_lo, m_hi, magic;
+};
+__device__ __forceinline__ DequantConsts dequant_consts() {
+    DequantConsts c{0x000F000Fu, 0x00F000F0u, 0x64006400u};
+    asm volatile("" : "+s"(c.m_lo), "+s"(c.m_hi), "+v"(c.magic));
+    return c;
+}
+
 // 4 words (32 codes) of one lane -> 4 x 8 fp16 weights  (w = (code - zero) * scale).
 // The integer part of the zero point is folded into the exact integer step that removes the
 // 1024 (low nibbles) / 64 (high nibbles, pre-scaled by 16) offset of the fp16 bit trick, so
 // only the fractional part of the zero point is rounded.
-__device__ __forceinline__ void dequant_tile(const uint4_t raw, const uint32_t szbits, half8_t (&a)[4]) {
+__device__ __forceinline__ void dequant_tile(const DequantConsts &c, const uint4_t raw, const uint32_t szbits,
+                                             half8_t (&a)[4]) {
     const half2_t sz = as_half2(szbits);
     const half_t s = sz.x, z = sz.y;
     const half_t zi = __builtin_rintf16(z);
@@ -64,10 +83,10 @@ __device__ __forceinline__ void dequant_tile(const uint4_t raw, const uint32_t s
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const uint32_t x = w[j], xs = x >> 8;
-        const half2_t t0 = as_half2((x & 0x000F000Fu) | 0x64006400u);
-        const half2_t t1 = as_half2((x & 0x00F000F0u) | 0x64006400u);
-        const half2_t t2 = as_half2((xs & 0x000F000Fu) | 0x64006400u);
-        const half2_t t3 = as_half2((xs & 0x00F000F0u) | 0x64006400u);
+        const half2_t t0 = as_half2((x & c.m_lo) | c.magic);
+        const half2_t t1 = as_half2((x & c.m_hi) | c.magic);
+        const half2_t t2 = as_half2((xs & c.m_lo) | c.magic);
+        const half2_t t3 = as_half2((xs & c.m_hi) | c.magic);
         const half2_t q0 = t0 + CLO;
         const half2_t q1 = __builtin_elementwise_fma(t1, R16, CHI);
         const half2_t q2 = t2 + CLO;
@@ -82,15 +101,41 @@ __device__ __forceinline__ void dequant_tile(const uint4_t raw, const uint32_t s
 
 __device__ __forceinline__ float silu_f32(float g) { return g / (1.0f + __expf(-g)); }
 
-template <int NB, int MB, int MODE>
-__global__ __launch_bounds__(256) void w4_gemm_kernel(const GemmParams p) {
-    static_assert(MODE == 1 || NB % 2 == 0, "gate_up needs gate/up block pairs");
-    __shared__ __attribute__((aligned(16))) half_t xs[2][16 * MB][XS_STRIDE];
+// s_waitcnt vmcnt(N) only (gfx9 encoding: vmcnt = bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8)
+#define ODSD_WAIT_VMCNT(N) \
+    __builtin_amdgcn_s_waitcnt(((N) & 0xF) | (((N) >> 4) << 14) | (7 << 4) | (0xF << 8))
 
-    // workgroup -> (expert, row chunk, k split); consecutive logical ids share an XCD so
-    // that one expert's token rows stay in one L2
+typedef __attribute__((address_space(3))) void lds_void;
+
+// NB    16-row weight blocks per wavefront          MB  16-row token blocks per pass
+// DEPTH groups of weight loads kept in flight       NA  blocks expanded to fp16 at a time
+// WK    wavefronts of a workgroup that split the reduction dimension among themselves
+//       (their partial sums are added through LDS in a fixed order at the end)
+// DIRECT == true  (MB == 1): token rows are never staged; each wavefront reads its B
+//       fragments straight from L1/L2 as part of the ring slot -- no barrier in the loop.
+// DIRECT == false (WK == 1): token rows go global -> LDS by asynchronous DMA loads
+//       (global_load_lds, no registers), three buffers deep, 16-byte segments XOR-swizzled
+//       by the row so that the B-fragment reads are bank-conflict free; one raw s_barrier
+//       per group, preceded by a vmcnt wait that leaves the newest loads in flight.
+template <int NB, int MB, int MODE, int DEPTH, int NA, int WK, bool DIRECT>
+__global__ __launch_bounds__(256, (MB >= 8 ? 1 : 2)) void w4_gemm_kernel(const GemmParams p) {
+    static_assert(MODE == 1 || NB % 2 == 0, "gate_up needs gate/up block pairs");
+    static_assert(NB % NA == 0, "NA must divide NB");
+    static_assert(!DIRECT || MB == 1, "the direct path holds one token block");
+    static_assert(DIRECT || WK == 1, "K is split across wavefronts on the direct path only");
+    constexpr int RSUB = 4 / WK;                  // wavefronts along the rows
+    constexpr int XS_BYTES = DIRECT ? 16 : 3 * 16 * MB * 256;
+    constexpr int RED_FLOATS = WK > 1 ? (WK - 1) * RSUB * 64 * NB * 4 : 1;
+    __shared__ __attribute__((aligned(16))) char xs_raw[XS_BYTES];
+    __shared__ __attribute__((aligned(16))) float red[RED_FLOATS];
+
+    // workgroup -> (expert, row chunk, k split).  Hardware deals workgroups round-robin over
+    // the 8 XCDs.  With many token rows per expert (MB >= 8) consecutive logical ids are kept
+    // on one XCD so that an expert's rows stay in one L2; with few rows that locality is worth
+    // nothing and would leave an XCD idle for every expert without tokens, so the chunks of
+    // one expert are spread over all XCDs instead.
     const int b = blockIdx.x;
-    const int L = (b & 7) * p.wg_per_xcd + (b >> 3);
+    const int L = MB >= 8 ? (b & 7) * p.wg_per_xcd + (b >> 3) : b;
     if (L >= p.n_wg) return;
     const int ks = L % p.KS;
     const int chunk = (L / p.KS) % p.nchunks;
@@ -100,22 +145,42 @@ __global__ __launch_bounds__(256) void w4_gemm_kernel(const GemmParams p) {
     if (M_e == 0) return;
     const uint64_t *trow = p.table + (size_t)e * ODSD_TABLE_COLS;
     if (trow[0] == 0) return;
-    const uint4_t *qp = (const uint4_t *)(MODE == 0 ? trow[0] : trow[2]);
-    const uint32_t *szp = (const uint32_t *)(MODE == 0 ? trow[1] : trow[3]);
+    // addresses from the table are global memory: say so, or the loads become flat loads
+    // whose LDS-side counter forces every wait to drain
+    const global_char *qp_c = (const global_char *)(MODE == 0 ? trow[0] : trow[2]);
+    const global_char *szp_c = (const global_char *)(MODE == 0 ? trow[1] : trow[3]);
+    const global_char *src_c = (const global_char *)p.src;
     const int base = p.offsets[e];
 
+    const DequantConsts dc = dequant_consts();
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int r = lane & 15, kq = lane >> 4;
-    const int g_begin = ks * p.gper;
-    const int g_end = min(p.G, g_begin + p.gper);
+    const int kpart = wave % WK, rsub = wave / WK;
+    // K range of the workgroup, then of this wavefront
+    const int G_begin = ks * p.gper;
+    const int G_end = min(p.G, G_begin + p.gper);
+    const int gw = (G_end - G_begin + WK - 1) / WK;
+    const int g_begin = G_begin + kpart * gw;
+    const int g_end = min(G_end, g_begin + gw);
+    const int g_last = max(g_end - 1, G_begin);
 
-    const int blk0 = (chunk * 4 + wave) * NB;   // first 16-row block of this wavefront
+    // Every load in the main loop is unconditional (out-of-range blocks and groups are
+    // clamped to a valid tile and their results never stored): straight-line code lets the
+    // hardware counters keep several groups of loads in flight instead of draining them.
+    // Addresses are a uniform base plus a 32-bit per-lane byte offset (one VGPR per load).
+    const int blk0 = (chunk * RSUB + rsub) * NB;   // first 16-row block of this wavefront
     bool blk_ok[NB];
+    uint32_t wq_off[NB], sz_off[NB];
 #pragma unroll
-    for (int i = 0; i < NB; ++i) blk_ok[i] = blk0 + i < p.NBLK;
+    for (int i = 0; i < NB; ++i) {
+        blk_ok[i] = blk0 + i < p.NBLK;
+        const uint32_t blk = blk_ok[i] ? blk0 + i : 0;
+        wq_off[i] = (blk * p.G * 64 + lane) * 16u;
+        sz_off[i] = (blk * p.G * 16 + r) * 4u;
+    }
 
-    // x staging: row = piece / 16, 16-byte segment = piece % 16, piece = tid + 256 i
+    // x staging (DMA path): piece = tid + 256 i -> row = piece / 16, segment = piece % 16
     const int st_seg = tid & 15;
     const int st_row0 = tid >> 4;
 
@@ -123,16 +188,19 @@ __global__ __launch_bounds__(256) void w4_gemm_kernel(const GemmParams p) {
         const int mcnt = min(M_e - m0, 16 * MB);
         const int nmb = (mcnt + 15) >> 4;
 
-        const half_t *st_src[MB];
+        // byte offsets of the token rows this thread fetches
+        //   DMA path:    piece i -> row st_row0 + 16 i, source segment st_seg ^ (row & 15)
+        //   DIRECT path: row r of the block, columns 8*kq.. of each 32-column step
+        // rows past the expert's last one are clamped to its first row: the MFMA columns they
+        // feed are never stored
+        uint32_t st_off[MB];
 #pragma unroll
         for (int i = 0; i < MB; ++i) {
-            const int row = st_row0 + 16 * i;
-            st_src[i] = nullptr;
-            if (row < mcnt) {
-                const int slot = base + m0 + row;
-                const int srow = p.rowmap ? p.rowmap[slot] : slot;
-                st_src[i] = p.src + (size_t)srow * p.src_ld + st_seg * 8;
-            }
+            const int row = DIRECT ? r : st_row0 + 16 * i;
+            const int slot = base + m0 + (row < mcnt ? row : 0);
+            const int srow = p.rowmap ? p.rowmap[slot] : slot;
+            const int seg = DIRECT ? kq : (st_seg ^ (row & 15));
+            st_off[i] = ((uint32_t)srow * (uint32_t)p.src_ld + seg * 8) * 2u;
         }
 
         float4_t acc[NB][MB];
@@ -141,83 +209,135 @@ __global__ __launch_bounds__(256) void w4_gemm_kernel(const GemmParams p) {
 #pragma unroll
             for (int m = 0; m < MB; ++m) acc[i][m] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-        uint4_t wq[2][NB];
-        uint32_t wsz[2][NB];
-        uint4_t xr[MB];
+        uint4_t wq[DEPTH][NB];
+        uint32_t wsz[DEPTH][NB];
+        uint4_t xd[DIRECT ? DEPTH : 1][4];   // DIRECT: B fragments travel with the ring slot
 
         auto load_w = [&](int buf, int g) {
+            const uint32_t gc = (uint32_t)min(g, g_last);
 #pragma unroll
             for (int i = 0; i < NB; ++i) {
-                if (blk_ok[i] && g < g_end) {
-                    const size_t tile = (size_t)(blk0 + i) * p.G + g;
-                    wq[buf][i] = __builtin_nontemporal_load(qp + tile * 64 + lane);
-                    wsz[buf][i] = szp[tile * 16 + r];
-                } else {
-                    wq[buf][i] = uint4_t{0, 0, 0, 0};
-                    wsz[buf][i] = 0;
-                }
+                wq[buf][i] = __builtin_nontemporal_load((const global_u4 *)(qp_c + (wq_off[i] + gc * 1024u)));
+                wsz[buf][i] = *(const global_u32 *)(szp_c + (sz_off[i] + gc * 64u));
             }
         };
-        auto load_x = [&](int g) {
+        // DIRECT: the B fragments of group g (refilled only after the products that read them)
+        auto load_xd = [&](int buf, int g) {
+            const uint32_t gc = (uint32_t)min(g, g_last);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                xd[DIRECT ? buf : 0][j] =
+                    *(const global_u4 *)(src_c + (st_off[0] + gc * (ODSD_GROUP * 2u) + j * 64u));
+        };
+        // MB asynchronous 16-byte loads per thread: global -> xs[buf] (no registers)
+        auto dma_x = [&](int buf, int g) {
+            const uint32_t gc = (uint32_t)min(g, g_last);
 #pragma unroll
             for (int i = 0; i < MB; ++i) {
-                if (st_src[i] != nullptr && i < nmb)
-                    xr[i] = *(const uint4_t *)(st_src[i] + (size_t)g * ODSD_GROUP);
-                else
-                    xr[i] = uint4_t{0, 0, 0, 0};
-            }
-        };
-        auto store_x = [&](int buf) {
-#pragma unroll
-            for (int i = 0; i < MB; ++i)
-                if (i < nmb) *(uint4_t *)&xs[buf][st_row0 + 16 * i][st_seg * 8] = xr[i];
-        };
-        auto compute = [&](int buf, int xbuf) {
-            half8_t a[NB][4];
-#pragma unroll
-            for (int i = 0; i < NB; ++i) dequant_tile(wq[buf][i], wsz[buf][i], a[i]);
-#pragma unroll
-            for (int m = 0; m < MB; ++m) {
-                if (m < nmb) {
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const half8_t bx = *(const half8_t *)&xs[xbuf][m * 16 + r][j * 32 + kq * 8];
-#pragma unroll
-                        for (int i = 0; i < NB; ++i)
-                            acc[i][m] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i][j], bx, acc[i][m], 0, 0, 0);
-                    }
-                }
+                lds_void *dst = (lds_void *)(xs_raw + buf * (16 * MB * 256) + (i * 256 + wave * 64) * 16);
+                __builtin_amdgcn_global_load_lds((const global_u4 *)(src_c + (st_off[i] + gc * (ODSD_GROUP * 2u))),
+                                                 dst, 16, 0, 0);
             }
         };
 
-        // software pipeline: weights two groups ahead in registers, x one group ahead
-        __syncthreads();   // previous pass is done with xs
-        load_x(g_begin);
-        load_w(0, g_begin);
-        load_w(1, g_begin + 1);
-        store_x(0);
-        __syncthreads();
-        for (int g = g_begin; g < g_end; g += 2) {
-            // even step: weights in buffer 0, x in xs[0]
-            if (g + 1 < g_end) load_x(g + 1);
-            compute(0, 0);
-            load_w(0, g + 2);
-            if (g + 1 < g_end) store_x(1);
+        if (!DIRECT) {
+            __builtin_amdgcn_s_barrier();   // the previous pass is done with xs
+            dma_x(0, g_begin);
+            dma_x(1, g_begin + 1);
+        }
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            load_w(d, g_begin + d);
+            if (DIRECT) load_xd(d, g_begin + d);
+        }
+        if (!DIRECT) {
+            // x(g_begin) has landed once at most the loads issued after it are outstanding
+            ODSD_WAIT_VMCNT(MB + DEPTH * 2 * NB);
+            __builtin_amdgcn_s_barrier();
+        }
+
+        int it = 0;
+        for (int g = g_begin; g < g_end;) {
+#pragma unroll
+            for (int d = 0; d < DEPTH; ++d) {
+                const int xb = it % 3;
+                if (!DIRECT) dma_x((it + 2) % 3, g + 2);
+                __builtin_amdgcn_sched_barrier(0);
+                half8_t bdir[4];
+                if (DIRECT) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) bdir[j] = __builtin_bit_cast(half8_t, xd[DIRECT ? d : 0][j]);
+                }
+                const char *xbase = xs_raw + xb * (16 * MB * 256);
+#pragma unroll
+                for (int h = 0; h < NB; h += NA) {
+                    half8_t a[NA][4];
+#pragma unroll
+                    for (int i = 0; i < NA; ++i) dequant_tile(dc, wq[d][h + i], wsz[d][h + i], a[i]);
+                    if (h + NA >= NB) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        load_w(d, g + DEPTH);      // ring slot d is free again
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+#pragma unroll
+                    for (int m = 0; m < MB; ++m) {
+                        if (m < nmb) {
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) {
+                                half8_t bx;
+                                if (DIRECT) {
+                                    bx = bdir[j];
+                                } else {
+                                    // row m*16 + r, logical segment 4j + kq, stored at segment ^ (row & 15)
+                                    const int seg = (4 * j + kq) ^ r;
+                                    bx = *(const half8_t *)(xbase + ((m * 16 + r) * 16 + seg) * 16);
+                                }
+#pragma unroll
+                                for (int i = 0; i < NA; ++i)
+                                    acc[h + i][m] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i][j], bx, acc[h + i][m], 0, 0, 0);
+                            }
+                        }
+                    }
+                }
+                if (DIRECT) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    load_xd(d, g + DEPTH);
+                } else {
+                    __builtin_amdgcn_sched_barrier(0);
+                    // x(g+1) was issued one step ago; the loads issued after it are that step's
+                    // refill, this step's DMA and this step's refill
+                    ODSD_WAIT_VMCNT(4 * NB + MB);
+                    __builtin_amdgcn_s_barrier();
+                }
+                ++g;
+                ++it;
+                if (g >= g_end) break;
+            }
+        }
+
+        if (WK > 1) {
+            // partial sums of the K parts: parts 1.. go through LDS, part 0 adds them in order
             __syncthreads();
-            if (g + 1 >= g_end) break;
-            // odd step: weights in buffer 1, x in xs[1]
-            if (g + 2 < g_end) load_x(g + 2);
-            compute(1, 1);
-            load_w(1, g + 3);
-            if (g + 2 < g_end) store_x(0);
+            if (kpart > 0) {
+#pragma unroll
+                for (int i = 0; i < NB; ++i)
+                    *(float4_t *)&red[(((kpart - 1) * RSUB + rsub) * NB + i) * 256 + lane * 4] = acc[i][0];
+            }
             __syncthreads();
+            if (kpart == 0) {
+#pragma unroll
+                for (int k = 1; k < WK; ++k)
+#pragma unroll
+                    for (int i = 0; i < NB; ++i)
+                        acc[i][0] += *(const float4_t *)&red[(((k - 1) * RSUB + rsub) * NB + i) * 256 + lane * 4];
+            }
         }
 
         // epilogue: lane holds rows 4*kq..4*kq+3 of each 16-row block, token column r
 #pragma unroll
         for (int m = 0; m < MB; ++m) {
             const int row = m * 16 + r;
-            if (m < nmb && row < mcnt) {
+            if (m < nmb && row < mcnt && kpart == 0) {
                 const size_t slot = (size_t)(base + m0 + row);
                 if (MODE == 0) {
 #pragma unroll
@@ -244,6 +364,7 @@ __global__ __launch_bounds__(256) void w4_gemm_kernel(const GemmParams p) {
                 }
             }
         }
+        if (WK > 1) __syncthreads();   // red is reused by the next pass
     }
 }
 
@@ -299,31 +420,48 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
 struct ExpertsPlan {
     int MB;          // 16-row token blocks held per pass
     int NB;          // 16-row weight blocks per wavefront
-    int KS;          // split of the down projection's reduction dimension
+    int WK_gu, WK_dn;  // wavefronts splitting K inside a workgroup (MB == 1 path)
+    int KS;          // split of the down projection's reduction dimension across workgroups
     size_t h_bytes, y_bytes;
 };
 
+// Choices are functions of the shape only (the per-expert counts live on the device).
 static ExpertsPlan experts_plan(const odsd_moe_shape *s) {
     ExpertsPlan p;
-    // rows one expert can receive is at most T (distinct ids per token); size the register
-    // tile for the common case and let rarer, larger experts take extra passes
     const long P = (long)s->T * s->K;
     const long mean_rows = (P + s->E - 1) / s->E;
     if (s->T <= 16) p.MB = 1;
     else if (s->T <= 32) p.MB = 2;
     else p.MB = (mean_rows * 3 / 2 <= 64) ? 4 : 8;
+    const long active = s->E < P ? s->E : P;       // upper bound of experts with rows
+    const long slots = 512;                        // 256 CUs x 2 workgroups
+    const int G_gu = s->H / ODSD_GROUP, G_dn = s->I / ODSD_GROUP;
     p.NB = 4;
-    // down projection: enough workgroups to cover the machine (~4 per CU)
-    const int nchunks_dn = (s->H / 16 + 4 * p.NB - 1) / (4 * p.NB);
-    const long active = s->E < P ? s->E : P;
-    const int G = s->I / ODSD_GROUP;
-    int KS = 1;
-    while (KS * 2 <= G && active * nchunks_dn * KS < 1024 && KS < 16) KS *= 2;
+    p.WK_gu = p.WK_dn = 1;
+    p.KS = 1;
+    if (p.MB == 1) {
+        // many small work items: 4 wavefronts split K when each still gets >= 2 groups
+        p.WK_gu = G_gu >= 8 ? 4 : (G_gu >= 4 ? 2 : 1);
+        const long chunks_dn = (s->H / 16 + 4 - 1) / 4;   // with WK = 4: 64 rows per workgroup
+        int KS = 1;
+        while (KS * 2 <= G_dn / 8 && active * chunks_dn * KS < 8 * slots && KS < 16) KS *= 2;
+        p.KS = KS;
+        const int gper = (G_dn + KS - 1) / KS;
+        p.WK_dn = gper >= 8 ? 4 : (gper >= 4 ? 2 : 1);
+    } else {
+        if (p.MB <= 4) {
+            const long wg_gu = active * ((2 * s->I / 16 + 15) / 16);
+            if (wg_gu < 4 * slots) p.NB = 2;
+        }
+        const int nchunks_dn = (s->H / 16 + 4 * p.NB - 1) / (4 * p.NB);
+        int KS = 1;
+        while (KS * 2 <= G_dn / 2 && active * nchunks_dn * KS < 4 * slots && KS < 16) KS *= 2;
+        p.KS = KS;
+    }
     // every split must own at least one group
-    while (KS > 1 && ((G + KS - 1) / KS) * (KS - 1) >= G) KS--;
-    p.KS = KS;
+    while (p.KS > 1 && ((G_dn + p.KS - 1) / p.KS) * (p.KS - 1) >= G_dn) p.KS--;
     p.h_bytes = odsd_round_up((size_t)(P > 0 ? P : 1) * s->I * sizeof(half_t), 256);
-    p.y_bytes = odsd_round_up((size_t)KS * (size_t)(P > 0 ? P : 1) * s->H * sizeof(float), 256);
+    p.y_bytes = odsd_round_up((size_t)p.KS * (size_t)(P > 0 ? P : 1) * s->H * sizeof(float), 256);
     return p;
 }
 
@@ -342,60 +480,95 @@ extern "C" size_t odsd_experts_workspace_bytes(const odsd_moe_shape *s) {
     return p.h_bytes + p.y_bytes;
 }
 
-template <int NB, int MB, int MODE>
+template <int NB, int MB, int MODE, int DEPTH, int NA, int WK, bool DIRECT>
 static void launch_gemm(GemmParams &gp, hipStream_t st) {
+    gp.nchunks = (gp.NBLK + (4 / WK) * NB - 1) / ((4 / WK) * NB);
+    gp.n_wg = gp.E * gp.nchunks * gp.KS;
     gp.wg_per_xcd = (gp.n_wg + 7) / 8;
-    w4_gemm_kernel<NB, MB, MODE><<<gp.wg_per_xcd * 8, 256, 0, st>>>(gp);
+    w4_gemm_kernel<NB, MB, MODE, DEPTH, NA, WK, DIRECT><<<gp.wg_per_xcd * 8, 256, 0, st>>>(gp);
 }
 
 template <int MODE>
-static void launch_gemm_mb(int MB, GemmParams &gp, hipStream_t st) {
-    switch (MB) {
-        case 1: launch_gemm<4, 1, MODE>(gp, st); break;
-        case 2: launch_gemm<4, 2, MODE>(gp, st); break;
-        case 4: launch_gemm<4, 4, MODE>(gp, st); break;
-        default: launch_gemm<4, 8, MODE>(gp, st); break;
+static void launch_gemm_plan(const ExpertsPlan &pl, GemmParams &gp, hipStream_t st) {
+    const int wk = MODE == 0 ? pl.WK_gu : pl.WK_dn;
+    if (pl.MB == 1) {
+        if (wk == 4) launch_gemm<4, 1, MODE, 2, 2, 4, true>(gp, st);
+        else if (wk == 2) launch_gemm<4, 1, MODE, 3, 2, 2, true>(gp, st);
+        else launch_gemm<4, 1, MODE, 3, 2, 1, true>(gp, st);
+    } else if (pl.MB == 2) {
+        if (pl.NB == 2) launch_gemm<2, 2, MODE, 3, 2, 1, false>(gp, st);
+        else launch_gemm<4, 2, MODE, 3, 4, 1, false>(gp, st);
+    } else if (pl.MB == 4) {
+        if (pl.NB == 2) launch_gemm<2, 4, MODE, 3, 2, 1, false>(gp, st);
+        else launch_gemm<4, 4, MODE, 2, 2, 1, false>(gp, st);
+    } else {
+        launch_gemm<4, 8, MODE, 2, 4, 1, false>(gp, st);
     }
 }
 
-int odsd_launch_experts(const odsd_moe_shape *s, const void *x16, const uint64_t *table, const int32_t *idx,
-                        const float *w, const int32_t *counts, const int32_t *offsets, const int32_t *perm,
-                        const int32_t *slot_token, const void *residual, float *out_f32, void *out_act,
-                        void *ws, size_t ws_bytes, hipStream_t st) {
+static int experts_args_ok(const odsd_moe_shape *s) {
     const int rc = experts_check(s);
+    return rc;
+}
+
+// gate_up + SiLU*mul: x_f16 [T,H] gathered by slot_token -> h_f16 [P,I] in slot order
+extern "C" int odsd_w4_gate_up_silu(const odsd_moe_shape *s, const void *x_f16, const uint64_t *table,
+                                    const int32_t *counts, const int32_t *offsets,
+                                    const int32_t *slot_token, void *h_f16, void *stream) {
+    const int rc = experts_args_ok(s);
     if (rc != ODSD_OK) return rc;
     if (s->T == 0) return ODSD_OK;
-    if (!x16 || !table || !idx || !w || !counts || !offsets || !perm || !slot_token || !ws)
-        return ODSD_ERR_NULL;
-    if (!out_f32 && !out_act) return ODSD_ERR_NULL;
-    if (!odsd_aligned16(x16) || !odsd_aligned16(ws) || (out_f32 && !odsd_aligned16(out_f32)))
-        return ODSD_ERR_ALIGN;
+    if (!x_f16 || !table || !counts || !offsets || !slot_token || !h_f16) return ODSD_ERR_NULL;
+    if (!odsd_aligned16(x_f16) || !odsd_aligned16(h_f16)) return ODSD_ERR_ALIGN;
     const ExpertsPlan pl = experts_plan(s);
-    if (ws_bytes < pl.h_bytes + pl.y_bytes) return ODSD_ERR_WORKSPACE;
-    half_t *h16 = (half_t *)ws;
-    float *y = (float *)((char *)ws + pl.h_bytes);
-    const int P = s->T * s->K;
-
     GemmParams gu{};
-    gu.table = table; gu.src = (const half_t *)x16; gu.rowmap = slot_token;
-    gu.counts = counts; gu.offsets = offsets; gu.h16 = h16; gu.y = nullptr;
+    gu.table = table; gu.src = (const half_t *)x_f16; gu.rowmap = slot_token;
+    gu.counts = counts; gu.offsets = offsets; gu.h16 = (half_t *)h_f16; gu.y = nullptr;
     gu.src_ld = s->H; gu.G = s->H / ODSD_GROUP; gu.NBLK = 2 * s->I / 16;
-    gu.nchunks = (gu.NBLK + 4 * pl.NB - 1) / (4 * pl.NB);
-    gu.KS = 1; gu.gper = gu.G; gu.ldo = s->I; gu.P = P;
-    gu.n_wg = s->E * gu.nchunks;
-    launch_gemm_mb<0>(pl.MB, gu, st);
+    gu.KS = 1; gu.gper = gu.G; gu.ldo = s->I; gu.P = s->T * s->K; gu.E = s->E;
+    launch_gemm_plan<0>(pl, gu, (hipStream_t)stream);
     ODSD_CHECK_LAUNCH();
+    return ODSD_OK;
+}
 
+extern "C" int32_t odsd_w4_down_splits(const odsd_moe_shape *s) {
+    if (experts_check(s) != ODSD_OK) return 0;
+    return experts_plan(s).KS;
+}
+
+// down: h_f16 [P,I] -> y [KS][P][H] fp32 partial sums over KS slices of I
+extern "C" int odsd_w4_down(const odsd_moe_shape *s, const void *h_f16, const uint64_t *table,
+                            const int32_t *counts, const int32_t *offsets, float *y, void *stream) {
+    const int rc = experts_args_ok(s);
+    if (rc != ODSD_OK) return rc;
+    if (s->T == 0) return ODSD_OK;
+    if (!h_f16 || !table || !counts || !offsets || !y) return ODSD_ERR_NULL;
+    if (!odsd_aligned16(h_f16) || !odsd_aligned16(y)) return ODSD_ERR_ALIGN;
+    const ExpertsPlan pl = experts_plan(s);
     GemmParams dn{};
-    dn.table = table; dn.src = h16; dn.rowmap = nullptr;
+    dn.table = table; dn.src = (const half_t *)h_f16; dn.rowmap = nullptr;
     dn.counts = counts; dn.offsets = offsets; dn.h16 = nullptr; dn.y = y;
     dn.src_ld = s->I; dn.G = s->I / ODSD_GROUP; dn.NBLK = s->H / 16;
-    dn.nchunks = (dn.NBLK + 4 * pl.NB - 1) / (4 * pl.NB);
-    dn.KS = pl.KS; dn.gper = (dn.G + pl.KS - 1) / pl.KS; dn.ldo = s->H; dn.P = P;
-    dn.n_wg = s->E * dn.nchunks * dn.KS;
-    launch_gemm_mb<1>(pl.MB, dn, st);
+    dn.KS = pl.KS; dn.gper = (dn.G + pl.KS - 1) / pl.KS; dn.ldo = s->H; dn.P = s->T * s->K; dn.E = s->E;
+    launch_gemm_plan<1>(pl, dn, (hipStream_t)stream);
     ODSD_CHECK_LAUNCH();
+    return ODSD_OK;
+}
 
+// combine: y partials + routing weights (+ residual) -> out
+extern "C" int odsd_combine(const odsd_moe_shape *s, const float *y, const int32_t *idx, const float *w,
+                            const int32_t *perm, const uint64_t *table, const void *residual,
+                            float *out_f32, void *out_act, void *stream) {
+    const int rc = experts_args_ok(s);
+    if (rc != ODSD_OK) return rc;
+    if (s->T == 0) return ODSD_OK;
+    if (!y || !idx || !w || !perm || !table) return ODSD_ERR_NULL;
+    if (!out_f32 && !out_act) return ODSD_ERR_NULL;
+    if (!odsd_aligned16(y) || (out_f32 && !odsd_aligned16(out_f32))) return ODSD_ERR_ALIGN;
+    if (s->T > 65535) return ODSD_ERR_UNSUPPORTED;
+    const ExpertsPlan pl = experts_plan(s);
+    const int P = s->T * s->K;
+    hipStream_t st = (hipStream_t)stream;
     const dim3 grid((s->H / 4 + 255) / 256, s->T);
     if (s->act_dtype == ODSD_DT_BF16)
         combine_kernel<uint16_t><<<grid, 256, 0, st>>>(y, idx, w, perm, table, (const uint16_t *)residual,
@@ -407,6 +580,26 @@ int odsd_launch_experts(const odsd_moe_shape *s, const void *x16, const uint64_t
                                                     pl.KS, P);
     ODSD_CHECK_LAUNCH();
     return ODSD_OK;
+}
+
+int odsd_launch_experts(const odsd_moe_shape *s, const void *x16, const uint64_t *table, const int32_t *idx,
+                        const float *w, const int32_t *counts, const int32_t *offsets, const int32_t *perm,
+                        const int32_t *slot_token, const void *residual, float *out_f32, void *out_act,
+                        void *ws, size_t ws_bytes, hipStream_t st) {
+    int rc = experts_check(s);
+    if (rc != ODSD_OK) return rc;
+    if (s->T == 0) return ODSD_OK;
+    if (!ws) return ODSD_ERR_NULL;
+    if (!odsd_aligned16(ws)) return ODSD_ERR_ALIGN;
+    const ExpertsPlan pl = experts_plan(s);
+    if (ws_bytes < pl.h_bytes + pl.y_bytes) return ODSD_ERR_WORKSPACE;
+    void *h16 = ws;
+    float *y = (float *)((char *)ws + pl.h_bytes);
+    rc = odsd_w4_gate_up_silu(s, x16, table, counts, offsets, slot_token, h16, st);
+    if (rc != ODSD_OK) return rc;
+    rc = odsd_w4_down(s, h16, table, counts, offsets, y, st);
+    if (rc != ODSD_OK) return rc;
+    return odsd_combine(s, y, idx, w, perm, table, residual, out_f32, out_act, st);
 }
 
 extern "C" int odsd_experts_w4(const odsd_moe_shape *s, const void *x_f16, const uint64_t *table,

@@ -271,3 +271,39 @@ def moe_forward(x: torch.Tensor, gate_weight: torch.Tensor, table: torch.Tensor,
     plan = MoeForwardPlan(T, H, gate_weight.shape[0], top_k, inter, renorm, x.dtype, x.device,
                           want_f32, want_act)
     return plan.run(x, gate_weight, table, norm_weight, eps, add_residual)
+
+
+class ExpertStages:
+    """The three expert kernels as separate calls on caller-held h / y buffers (what
+    odsd_experts_w4 runs back to back); used to time or inspect the stages one by one."""
+
+    def __init__(self, T: int, H: int, E: int, K: int, I: int, dtype: torch.dtype, device):
+        lib = _lib.load()
+        self.shape = make_shape(T, H, E, K, I, False, dtype)
+        self.splits = lib.odsd_w4_down_splits(C.byref(self.shape))
+        if self.splits <= 0:
+            raise _lib.OdsdError(f"experts: unsupported shape T={T} H={H} E={E} K={K} I={I}")
+        P = max(T * K, 1)
+        self.h16 = torch.empty(P, I, dtype=torch.float16, device=device)
+        self.y = torch.empty(self.splits, P, H, dtype=torch.float32, device=device)
+
+    def gate_up(self, x_f16, table, disp: Dispatch) -> torch.Tensor:
+        lib = _lib.load()
+        _lib.check(lib.odsd_w4_gate_up_silu(C.byref(self.shape), x_f16.data_ptr(), table.data_ptr(),
+                                            disp.counts.data_ptr(), disp.offsets.data_ptr(),
+                                            disp.slot_token.data_ptr(), self.h16.data_ptr(), _stream()),
+                   "odsd_w4_gate_up_silu")
+        return self.h16
+
+    def down(self, table, disp: Dispatch) -> torch.Tensor:
+        lib = _lib.load()
+        _lib.check(lib.odsd_w4_down(C.byref(self.shape), self.h16.data_ptr(), table.data_ptr(),
+                                    disp.counts.data_ptr(), disp.offsets.data_ptr(), self.y.data_ptr(),
+                                    _stream()), "odsd_w4_down")
+        return self.y
+
+    def combine(self, idx, w, disp: Dispatch, table, residual=None, out_f32=None, out_act=None):
+        lib = _lib.load()
+        _lib.check(lib.odsd_combine(C.byref(self.shape), self.y.data_ptr(), idx.data_ptr(), w.data_ptr(),
+                                    disp.perm.data_ptr(), table.data_ptr(), _ptr(residual), _ptr(out_f32),
+                                    _ptr(out_act), _stream()), "odsd_combine")

@@ -1,0 +1,68 @@
+"""The C-ABI library loads without a GPU, exports every function the header declares, and
+rejects bad arguments with status codes before touching the device (CPU only)."""
+import ctypes as C
+import os
+import re
+
+from on_device_sd_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "odsd_moe.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(odsd_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_bound():
+    lib = _lib.load()
+    names = _declared()
+    assert len(names) >= 18
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in the header but not exported"
+        assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
+    assert sorted(_lib.SIGNATURES) == names
+
+
+def test_version_and_status_strings():
+    lib = _lib.load()
+    assert lib.odsd_version() == 100
+    assert lib.odsd_status_string(0) == b"ok"
+    for code in range(1, 8):
+        assert len(lib.odsd_status_string(code)) > 3
+
+
+def test_argument_checks_need_no_gpu():
+    lib = _lib.load()
+    ok = _lib.MoeShape(8, 256, 8, 2, 256, 1, _lib.DT_BF16, 0)
+    assert lib.odsd_moe_workspace_bytes(C.byref(ok)) > 0
+    assert lib.odsd_router_workspace_bytes(C.byref(ok)) > 0
+    assert lib.odsd_experts_workspace_bytes(C.byref(ok)) > 0
+    assert lib.odsd_w4_down_splits(C.byref(ok)) >= 1
+    bad_h = _lib.MoeShape(8, 200, 8, 2, 256, 1, _lib.DT_BF16, 0)      # H % 128 != 0
+    assert lib.odsd_moe_workspace_bytes(C.byref(bad_h)) == 0
+    big_e = _lib.MoeShape(8, 256, 1024, 2, 256, 1, _lib.DT_BF16, 0)   # E > 512
+    assert lib.odsd_router_workspace_bytes(C.byref(big_e)) == 0
+    k_gt_e = _lib.MoeShape(8, 256, 4, 8, 256, 1, _lib.DT_BF16, 0)
+    assert lib.odsd_router_workspace_bytes(C.byref(k_gt_e)) == 0
+    # NULL pointers and bad shapes come back as status codes, nothing is launched
+    assert lib.odsd_w4_quantize(None, 0, 16, 128, None, None, None, None) == 1
+    assert lib.odsd_w4_quantize(1 << 20, 0, 16, 100, 1 << 20, 1 << 20, 1 << 20, None) == 2
+    assert lib.odsd_w4_quantize(1 << 20, 9, 16, 128, 1 << 20, 1 << 20, 1 << 20, None) == 7
+    assert lib.odsd_w4_pack(None, None, None, 16, 128, 1, 0, None, None, None) == 1
+    assert lib.odsd_w4_pack(1 << 20, 1 << 20, 1 << 20, 10, 128, 1, 0, 1 << 20, 1 << 20, None) == 2
+    assert lib.odsd_rmsnorm(None, None, 1, 4, 128, 1e-6, None, None) == 1
+    assert lib.odsd_router_topk(C.byref(ok), None, None, None, None, None, None, None, 0, None) == 1
+    assert lib.odsd_router_topk(C.byref(ok), 1 << 20, 1 << 20, 1 << 20, 1 << 20, None, None, 1 << 20, 16, None) == 5
+    assert lib.odsd_router_topk(C.byref(ok), (1 << 20) + 4, 1 << 20, 1 << 20, 1 << 20, None, None, 1 << 20, 1 << 30, None) == 4
+    assert lib.odsd_dispatch(C.byref(ok), None, None, None, None, None, None, None) == 1
+    assert lib.odsd_moe_forward(C.byref(bad_h), None, None, 1e-6, None, None, 0, None, None, None, None, None,
+                                None, None, None, 0, None) == 2
+    assert lib.odsd_moe_forward(C.byref(ok), 1 << 20, None, 1e-6, 1 << 20, 1 << 20, 0, None, None, None, None,
+                                None, None, None, 1 << 20, 16, None) == 5
+    assert lib.odsd_w4_packed_q_bytes(32, 256) == 32 * 256 // 2
+    assert lib.odsd_w4_packed_sz_bytes(32, 256) == 32 * 2 * 4
+    assert lib.odsd_w4_packed_q_bytes(30, 256) == 0
+    empty = _lib.MoeShape(0, 256, 8, 2, 256, 1, _lib.DT_BF16, 0)       # T == 0 is a no-op
+    assert lib.odsd_dispatch(C.byref(empty), 1 << 20, 1 << 20, 1 << 20, 1 << 20, 1 << 20, 1 << 20, None) == 0

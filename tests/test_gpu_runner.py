@@ -1,0 +1,179 @@
+"""The runner behind the reference's ModelRunner MoE interface (GPU).  The cases mirror the
+reference's own tests: demo/tests/unit/test_routing.py, test_forward_moe.py and the MoE part
+of test_engine_optimizations.py (:608-750)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_oracle as orc
+from tests.helpers import canon_to_oracle, check_output
+
+pytestmark = pytest.mark.gpu
+
+H, I, E, K, L = 256, 128, 4, 2, 2      # the reference's small_config scaled to the W4 rules
+
+
+@pytest.fixture(scope="module")
+def runner(dev):
+    import on_device_sd_amd as odsd
+    cfg = odsd.MoEConfig(hidden_size=H, num_hidden_layers=L, num_experts=E, num_experts_per_token=K,
+                         moe_intermediate_size=I, torch_dtype="bfloat16")
+    g = torch.Generator().manual_seed(0)
+    gates, banks, oracles = [], [], []
+    for l in range(L):
+        gates.append(torch.randn(E, H, generator=g) * 0.02)
+        bank = odsd.W4ExpertBank(E, H, I, dev)
+        ex = {}
+        for e in range(E):
+            canon = bank.load_expert(e, torch.randn(I, H, generator=g) * 0.02,
+                                     torch.randn(I, H, generator=g) * 0.02,
+                                     torch.randn(H, I, generator=g) * 0.02, keep_canonical=True)
+            ex[e] = canon_to_oracle(canon)
+        banks.append(bank)
+        oracles.append(ex)
+    norms = [torch.ones(H) for _ in range(L)]
+    r = odsd.W4MoERunner(cfg, gates, banks, norms)
+    r.oracle_experts = oracles
+    return r
+
+
+def _hidden(dev, *shape, seed=1):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g).to(torch.bfloat16).to(dev)
+
+
+def test_route_experts_output_format(runner, dev):
+    import on_device_sd_amd as odsd
+    hidden = _hidden(dev, 1, 4, H)
+    res = runner.route_experts(layer_idx=0, hidden_states=hidden)
+    assert isinstance(res, odsd.RoutingResult) and res.layer_idx == 0
+    assert res.topk_indices.shape[-1] == K and res.topk_scores.shape == res.topk_indices.shape
+    assert res.topk_indices.dtype == torch.int64 and res.top_k == K
+
+
+def test_routing_scores_sum_to_one(runner, dev):
+    res = runner.route_experts(0, _hidden(dev, 1, 4, H))
+    sums = res.topk_scores.sum(dim=-1)
+    assert torch.allclose(sums, torch.ones_like(sums), atol=1e-5)
+
+
+def test_activated_expert_ids_consistency(runner, dev):
+    import on_device_sd_amd as odsd
+    res = runner.route_experts(1, _hidden(dev, 9, H))          # 2-D input is accepted too
+    expected = {odsd.ExpertID(1, i) for i in res.topk_indices.flatten().unique().tolist()}
+    assert res.activated_expert_ids == expected
+
+
+def _attn(hidden):
+    import on_device_sd_amd as odsd
+    return odsd.AttentionOutput(hidden_states=hidden, post_attn_normed=hidden, residual=hidden)
+
+
+def _routing(layer, idx, scores):
+    import on_device_sd_amd as odsd
+    act = {odsd.ExpertID(layer, i) for i in idx.flatten().unique().tolist()}
+    return odsd.RoutingResult(layer_idx=layer, topk_indices=idx, topk_scores=scores, activated_expert_ids=act)
+
+
+def test_forward_moe_output_shape_and_values(runner, dev):
+    import on_device_sd_amd as odsd
+    hidden = _hidden(dev, 1, 2, H)
+    idx = torch.tensor([[0, 1], [1, 0]], device=dev)
+    scores = torch.full(idx.shape, 0.5, dtype=torch.float32, device=dev)
+    placement = odsd.ExpertPlacement(
+        gpu_expert_params={0: runner.banks[0].expert_params(0), 1: runner.banks[0].expert_params(1)},
+        cpu_expert_params={}, routing_result=_routing(0, idx, scores))
+    out = runner.forward_moe(0, _attn(hidden), placement)
+    assert out.shape == hidden.shape and out.dtype == hidden.dtype and out.abs().sum() > 0
+    flat = hidden.reshape(-1, H).cpu()
+    ref = orc.forward_moe(flat, flat, idx.cpu().numpy(), scores.cpu().numpy(), runner.oracle_experts[0])
+    check_output(out.reshape(-1, H), ref)
+
+
+def test_substitution_uses_substitute_params(runner, dev):
+    import on_device_sd_amd as odsd
+    hidden = _hidden(dev, 1, 2, H)
+    idx = torch.tensor([[1, 1], [1, 3]], device=dev)        # expert 3 is neither placed nor mapped
+    scores = torch.ones(idx.shape, dtype=torch.float32, device=dev)
+    placement = odsd.ExpertPlacement(gpu_expert_params={0: runner.banks[0].expert_params(0)},
+                                     cpu_expert_params={}, substitution_map={1: 0},
+                                     routing_result=_routing(0, idx, scores))
+    out = runner.forward_moe(0, _attn(hidden), placement)
+    flat = hidden.reshape(-1, H).cpu()
+    ref = orc.forward_moe(flat, flat, idx.cpu().numpy(), scores.cpu().numpy(),
+                          {0: runner.oracle_experts[0][0]}, substitution={1: 0})
+    check_output(out.reshape(-1, H), ref)
+    assert out.abs().sum() > 0
+
+
+def test_empty_routing_gives_zero_moe_contribution(runner, dev):
+    import on_device_sd_amd as odsd
+    hidden = _hidden(dev, 2, H)
+    placement = odsd.ExpertPlacement(gpu_expert_params={}, cpu_expert_params={}, routing_result=None)
+    out = runner.forward_moe(0, _attn(hidden), placement)
+    assert torch.equal(out, hidden)                          # residual + zeros
+    z = runner._execute_moe_with_placement(hidden, placement)
+    assert torch.equal(z, torch.zeros_like(hidden))
+
+
+def test_top1_weight_one_is_plain_expert_output(runner, dev):
+    import on_device_sd_amd as odsd
+    hidden = _hidden(dev, 3, H)
+    idx = torch.tensor([[0], [1], [2]], device=dev)
+    scores = torch.ones(3, 1, dtype=torch.float32, device=dev)
+    placement = odsd.ExpertPlacement(gpu_expert_params=runner.banks[0].all_expert_params(),
+                                     cpu_expert_params={}, routing_result=_routing(0, idx, scores))
+    moe = runner._execute_moe_with_placement(hidden, placement)
+    for t in range(3):
+        single = odsd.expert_forward_with_weights(hidden[t:t + 1], runner.banks[0].expert_params(t),
+                                                  return_f32=True)
+        ref = orc.expert_forward(hidden[t:t + 1].cpu(), *runner.oracle_experts[0][t].dequant())
+        check_output(single, ref)
+        assert torch.equal(moe[t], single[0].to(torch.bfloat16))
+
+
+def test_cpu_placed_fp_weights_are_refused(runner, dev):
+    import on_device_sd_amd as odsd
+    hidden = _hidden(dev, 2, H)
+    idx = torch.tensor([[0, 1], [0, 1]], device=dev)
+    scores = torch.ones(idx.shape, dtype=torch.float32, device=dev)
+    cpu_params = {"gate_proj": torch.zeros(I, H), "up_proj": torch.zeros(I, H), "down_proj": torch.zeros(H, I)}
+    placement = odsd.ExpertPlacement(gpu_expert_params={0: runner.banks[0].expert_params(0)},
+                                     cpu_expert_params={1: cpu_params}, routing_result=_routing(0, idx, scores))
+    with pytest.raises(TypeError, match="no CPU expert path"):
+        runner.forward_moe(0, _attn(hidden), placement)
+
+
+def test_route_then_forward_equals_whole_block_and_oracle(runner, dev):
+    import on_device_sd_amd as odsd
+    hidden = _hidden(dev, 2, 5, H, seed=3)
+    res = runner.route_experts(1, hidden)
+    placement = odsd.ExpertPlacement(gpu_expert_params=runner.banks[1].all_expert_params(),
+                                     cpu_expert_params={}, routing_result=res)
+    out = runner.forward_moe(1, _attn(hidden), placement)
+    flat = hidden.reshape(-1, H)
+    layer = odsd.moe_layer_forward(hidden, runner.gate_weights[1], runner.banks[1].all_expert_params(), E, K, I)
+    assert layer.shape == hidden.shape
+    assert torch.equal((flat.float() + layer.reshape(-1, H).float()).to(torch.bfloat16), out.reshape(-1, H))
+    ref, idx_o, _ = orc.moe_block(flat.cpu(), runner.gate_weights[1].cpu(), runner.oracle_experts[1], K, True)
+    assert np.array_equal(res.topk_indices.cpu().numpy(), idx_o.astype(np.int64))
+    check_output(odsd.moe_layer_forward(hidden, runner.gate_weights[1], runner.banks[1].all_expert_params(),
+                                        E, K, I, return_f32=True).reshape(-1, H), ref)
+
+
+def test_forward_layer_metadata_and_wiring(runner, dev):
+    hidden = _hidden(dev, 6, H, seed=4)
+    lo = runner.forward_layer(0, hidden)
+    assert lo.metadata == {"gpu_expert_count": E, "cpu_expert_count": 0, "substituted_count": 0}
+    out_o, _, _, _ = orc.moe_only_layer(hidden.cpu(), torch.ones(H, dtype=torch.bfloat16),
+                                        runner.gate_weights[0].cpu(), runner.oracle_experts[0], K, True)
+    d = (lo.hidden_states.cpu().float() - out_o.float()).abs()
+    assert d.max().item() <= 0.04 and d.mean().item() <= 2e-3
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    from on_device_sd_amd import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libodsd_moe.so")
+    with pytest.raises(ImportError, match="no\\s+CPU or PyTorch fallback"):
+        _lib.load()

@@ -1,0 +1,68 @@
+"""Host-side pieces that need no GPU: workload recipes, config sizes, data types."""
+import numpy as np
+import pytest
+import torch
+
+import on_device_sd_amd as odsd
+from on_device_sd_amd.workloads import CONFIGS, LayerInputs
+
+
+def test_workload_shapes_match_the_benchmark_configs():
+    c = CONFIGS
+    assert (c["tiny"].T, c["tiny"].H, c["tiny"].E, c["tiny"].K, c["tiny"].I) == (32, 512, 8, 2, 1024)
+    assert c["tiny"].act_dtype == torch.float32 and not c["tiny"].renorm
+    assert (c["mixtral_t160"].H, c["mixtral_t160"].E, c["mixtral_t160"].I) == (4096, 8, 14336)
+    assert c["qwen3_30b_t64_zipf"].renorm and c["qwen3_30b_t64_zipf"].zipf_s == 1.1
+    assert c["qwen3_30b_stack48_t256"].layers == 48
+    assert c["qwen3_235b_t4096"].regime == "prefill"
+    # per-expert bytes = 1.59375 * H * I
+    for w in c.values():
+        assert w.expert_w4_bytes == int(1.59375 * w.H * w.I)
+    assert abs(c["mixtral_t160"].E * c["mixtral_t160"].expert_w4_bytes / 1e6 - 748.7) < 0.1
+    assert abs(48 * 128 * c["qwen3_30b_stack48_t256"].expert_w4_bytes / 1e9 - 15.40) < 0.01
+    assert c["qwen3_235b_t4096"].algorithmic_flops() == 2 * 4096 * 4096 * 128 + 6 * 4096 * 8 * 4096 * 1536
+
+
+def test_layer_inputs_are_seeded_and_ordered():
+    wl = CONFIGS["tiny"]
+    a, b = LayerInputs(wl, "cpu"), LayerInputs(wl, "cpu")
+    ga, gb = a.gate_weight(), b.gate_weight()
+    assert torch.equal(ga, gb) and ga.shape == (8, 512) and ga.dtype == torch.float32
+    ea = next(iter(a.experts()))
+    eb = next(iter(b.experts()))
+    assert all(torch.equal(x, y) for x, y in zip(ea[1:], eb[1:]))
+    assert ea[1].shape == (1024, 512) and ea[3].shape == (512, 1024)
+    with pytest.raises(AssertionError):
+        LayerInputs(wl, "cpu").x()               # out of order
+    assert abs(float(ga.std()) - 0.02) < 2e-3
+
+
+def test_zipf_router_bias_skews_popularity():
+    wl = CONFIGS["qwen3_30b_t64_zipf"]
+    inp = LayerInputs(wl, "cpu")
+    gate = inp.gate_weight().float()
+    x = torch.randn(2000, wl.H, generator=torch.Generator().manual_seed(1)) + 8.0 / wl.H ** 0.5
+    top = torch.topk(x @ gate.t(), wl.K, dim=-1).indices
+    counts = np.sort(np.bincount(top.reshape(-1).numpy(), minlength=wl.E))[::-1]
+    assert counts[0] > 10 * max(counts[wl.E // 2], 1)        # strongly imbalanced
+    assert (counts > 0).sum() > wl.E // 2                    # but most experts still get tokens
+
+
+def test_config_and_ids():
+    cfg = odsd.MoEConfig()
+    assert cfg.get_dtype() == torch.bfloat16 and cfg.is_moe
+    assert cfg.get_expert_weight_size_bytes() == int(1.59375 * 2048 * 768)
+    a, b = odsd.ExpertID(1, 2), odsd.ExpertID(1, 2)
+    assert a == b and hash(a) == hash(b) and str(a) == "L1_E2" and len({a, b}) == 1
+    r = odsd.RoutingResult(0, torch.zeros(3, 2, dtype=torch.int64), torch.zeros(3, 2), set())
+    assert r.top_k == 2 and r.dispatch is None
+    p = odsd.ExpertPlacement(gpu_expert_params={}, cpu_expert_params={})
+    assert p.substitution_map == {} and p.routing_result is None
+
+
+def test_cpu_tensors_are_refused():
+    from on_device_sd_amd import ops
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ops.router_topk(torch.zeros(4, 128), torch.zeros(8, 128), 2, True)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ops.w4_quantize(torch.zeros(16, 128))
