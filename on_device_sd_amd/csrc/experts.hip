@@ -117,8 +117,8 @@ typedef __attribute__((address_space(3))) void lds_void;
 //       (global_load_lds, no registers), three buffers deep, 16-byte segments XOR-swizzled
 //       by the row so that the B-fragment reads are bank-conflict free; one raw s_barrier
 //       per group, preceded by a vmcnt wait that leaves the newest loads in flight.
-template <int NB, int MB, int MODE, int DEPTH, int NA, int WK, bool DIRECT>
-__global__ __launch_bounds__(256, (MB >= 8 ? 1 : 2)) void w4_gemm_kernel(const GemmParams p) {
+template <int NB, int MB, int MODE, int DEPTH, int NA, int WK, bool DIRECT, int OCC>
+__global__ __launch_bounds__(256, OCC) void w4_gemm_kernel(const GemmParams p) {
     static_assert(MODE == 1 || NB % 2 == 0, "gate_up needs gate/up block pairs");
     static_assert(NB % NA == 0, "NA must divide NB");
     static_assert(!DIRECT || MB == 1, "the direct path holds one token block");
@@ -422,12 +422,16 @@ struct ExpertsPlan {
     int NB;          // 16-row weight blocks per wavefront
     int WK_gu, WK_dn;  // wavefronts splitting K inside a workgroup (MB == 1 path)
     int KS;          // split of the down projection's reduction dimension across workgroups
+    int variant;     // tuning knob (environment ODSD_GEMM_VARIANT), 0 = default
     size_t h_bytes, y_bytes;
 };
 
 // Choices are functions of the shape only (the per-expert counts live on the device).
 static ExpertsPlan experts_plan(const odsd_moe_shape *s) {
     ExpertsPlan p;
+    static const int env_variant = getenv("ODSD_GEMM_VARIANT") ? atoi(getenv("ODSD_GEMM_VARIANT")) : 0;
+    static const int env_nb = getenv("ODSD_GEMM_NB") ? atoi(getenv("ODSD_GEMM_NB")) : 0;
+    p.variant = env_variant;
     const long P = (long)s->T * s->K;
     const long mean_rows = (P + s->E - 1) / s->E;
     if (s->T <= 16) p.MB = 1;
@@ -452,6 +456,7 @@ static ExpertsPlan experts_plan(const odsd_moe_shape *s) {
         if (p.MB <= 4) {
             const long wg_gu = active * ((2 * s->I / 16 + 15) / 16);
             if (wg_gu < 4 * slots) p.NB = 2;
+            if (env_nb == 2 || env_nb == 4) p.NB = env_nb;
         }
         const int nchunks_dn = (s->H / 16 + 4 * p.NB - 1) / (4 * p.NB);
         int KS = 1;
@@ -480,29 +485,34 @@ extern "C" size_t odsd_experts_workspace_bytes(const odsd_moe_shape *s) {
     return p.h_bytes + p.y_bytes;
 }
 
-template <int NB, int MB, int MODE, int DEPTH, int NA, int WK, bool DIRECT>
+template <int NB, int MB, int MODE, int DEPTH, int NA, int WK, bool DIRECT, int OCC>
 static void launch_gemm(GemmParams &gp, hipStream_t st) {
     gp.nchunks = (gp.NBLK + (4 / WK) * NB - 1) / ((4 / WK) * NB);
     gp.n_wg = gp.E * gp.nchunks * gp.KS;
     gp.wg_per_xcd = (gp.n_wg + 7) / 8;
-    w4_gemm_kernel<NB, MB, MODE, DEPTH, NA, WK, DIRECT><<<gp.wg_per_xcd * 8, 256, 0, st>>>(gp);
+    w4_gemm_kernel<NB, MB, MODE, DEPTH, NA, WK, DIRECT, OCC><<<gp.wg_per_xcd * 8, 256, 0, st>>>(gp);
 }
 
 template <int MODE>
 static void launch_gemm_plan(const ExpertsPlan &pl, GemmParams &gp, hipStream_t st) {
     const int wk = MODE == 0 ? pl.WK_gu : pl.WK_dn;
     if (pl.MB == 1) {
-        if (wk == 4) launch_gemm<4, 1, MODE, 2, 2, 4, true>(gp, st);
-        else if (wk == 2) launch_gemm<4, 1, MODE, 3, 2, 2, true>(gp, st);
-        else launch_gemm<4, 1, MODE, 3, 2, 1, true>(gp, st);
+        if (wk == 4) launch_gemm<4, 1, MODE, 2, 2, 4, true, 2>(gp, st);
+        else if (wk == 2) launch_gemm<4, 1, MODE, 3, 2, 2, true, 2>(gp, st);
+        else launch_gemm<4, 1, MODE, 3, 2, 1, true, 2>(gp, st);
     } else if (pl.MB == 2) {
-        if (pl.NB == 2) launch_gemm<2, 2, MODE, 3, 2, 1, false>(gp, st);
-        else launch_gemm<4, 2, MODE, 3, 4, 1, false>(gp, st);
+        if (pl.NB == 2) launch_gemm<2, 2, MODE, 3, 2, 1, false, 3>(gp, st);
+        else launch_gemm<4, 2, MODE, 3, 4, 1, false, 2>(gp, st);
     } else if (pl.MB == 4) {
-        if (pl.NB == 2) launch_gemm<2, 4, MODE, 3, 2, 1, false>(gp, st);
-        else launch_gemm<4, 4, MODE, 2, 2, 1, false>(gp, st);
+        if (pl.NB == 2) {
+            if (pl.variant == 1) launch_gemm<2, 4, MODE, 3, 2, 1, false, 2>(gp, st);
+            else if (pl.variant == 2) launch_gemm<2, 4, MODE, 3, 2, 1, false, 3>(gp, st);
+            else launch_gemm<2, 4, MODE, 2, 2, 1, false, 3>(gp, st);
+        } else {
+            launch_gemm<4, 4, MODE, 2, 2, 1, false, 2>(gp, st);
+        }
     } else {
-        launch_gemm<4, 8, MODE, 2, 4, 1, false>(gp, st);
+        launch_gemm<4, 8, MODE, 2, 4, 1, false, 1>(gp, st);
     }
 }
 

@@ -40,7 +40,7 @@ template <> struct Row8<float> {
 };
 
 // unit = (token tile, expert group, k split); 4 units (wavefronts) per workgroup.
-template <typename XT, int NE>
+template <typename XT, int NE, bool REDUCE4>
 __global__ __launch_bounds__(256) void router_partial_kernel(const XT *__restrict__ x,
                                                              const XT *__restrict__ wg,
                                                              double *__restrict__ partial,
@@ -114,6 +114,36 @@ __global__ __launch_bounds__(256) void router_partial_kernel(const XT *__restric
         }
     }
 
+    // When the K slices come in fours, the 4 wavefronts of this workgroup hold 4 consecutive
+    // slices of the same tile: add them through LDS in slice order and write one partial.
+    int s_out = s, S_out = S;
+    if (REDUCE4) {
+        __shared__ double red[3][NE][4][64];
+        const int wave = threadIdx.x >> 6;
+        if (wave > 0) {
+#pragma unroll
+            for (int i = 0; i < NE; ++i) {
+                red[wave - 1][i][0][lane] = acc[i].x;
+                red[wave - 1][i][1][lane] = acc[i].y;
+                red[wave - 1][i][2][lane] = acc[i].z;
+                red[wave - 1][i][3][lane] = acc[i].w;
+            }
+        }
+        __syncthreads();
+        if (wave > 0) return;
+#pragma unroll
+        for (int w = 0; w < 3; ++w)
+#pragma unroll
+            for (int i = 0; i < NE; ++i) {
+                acc[i].x += red[w][i][0][lane];
+                acc[i].y += red[w][i][1][lane];
+                acc[i].z += red[w][i][2][lane];
+                acc[i].w += red[w][i][3][lane];
+            }
+        s_out = s >> 2;
+        S_out = S >> 2;
+    }
+    (void)S_out;
 #pragma unroll
     for (int i = 0; i < NE; ++i) {
         const double v[4] = {acc[i].x, acc[i].y, acc[i].z, acc[i].w};
@@ -121,7 +151,7 @@ __global__ __launch_bounds__(256) void router_partial_kernel(const XT *__restric
         for (int q = 0; q < 4; ++q) {
             const int tq = tt * 16 + di[q];
             const int eq = (eg * NE + i) * 16 + dj[q];
-            if (tq < T && eq < E) partial[((size_t)s * T + tq) * E + eq] = v[q];
+            if (tq < T && eq < E) partial[((size_t)s_out * T + tq) * E + eq] = v[q];
         }
     }
 }
@@ -145,15 +175,27 @@ __global__ __launch_bounds__(256) void router_topk_kernel(const double *__restri
     double lg[ROUTER_MAX_V];
     uint64_t key[ROUTER_MAX_V];
     uint32_t taken = 0;   // bit v set: expert lane + 64 v already selected
+    // partial sums in slice order; the loads of one slice batch are independent of each other
+#pragma unroll
+    for (int v = 0; v < ROUTER_MAX_V; ++v) lg[v] = 0.0;
+    for (int s0 = 0; s0 < S; s0 += 4) {
+        double part[4][ROUTER_MAX_V];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int v = 0; v < ROUTER_MAX_V; ++v) {
+                const int e = lane + 64 * v;
+                part[u][v] = (e < E && s0 + u < S) ? partial[((size_t)(s0 + u) * T + t) * E + e] : 0.0;
+            }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int v = 0; v < ROUTER_MAX_V; ++v) lg[v] += part[u][v];
+    }
 #pragma unroll
     for (int v = 0; v < ROUTER_MAX_V; ++v) {
-        const int e = lane + 64 * v;
-        double a = 0.0;
-        if (e < E)
-            for (int s = 0; s < S; ++s) a += partial[((size_t)s * T + t) * E + e];
-        lg[v] = a;
-        key[v] = order_key(a);
-        if (e >= E) taken |= 1u << v;
+        key[v] = order_key(lg[v]);
+        if (lane + 64 * v >= E) taken |= 1u << v;
     }
 
     int my_e = 0;          // lane k keeps the k-th winner
@@ -252,8 +294,12 @@ template <typename XT, int NE>
 static void launch_partial(const RouterPlan &p, const odsd_moe_shape *s, const void *x, const void *gw,
                            double *partial, void *x16, hipStream_t st) {
     const int n_units = p.TT * p.EG * p.S;
-    router_partial_kernel<XT, NE><<<(n_units + 3) / 4, 256, 0, st>>>(
-        (const XT *)x, (const XT *)gw, partial, (half_t *)x16, s->T, s->H, s->E, p.S, p.EG, n_units);
+    if (p.S % 4 == 0)
+        router_partial_kernel<XT, NE, true><<<n_units / 4, 256, 0, st>>>(
+            (const XT *)x, (const XT *)gw, partial, (half_t *)x16, s->T, s->H, s->E, p.S, p.EG, n_units);
+    else
+        router_partial_kernel<XT, NE, false><<<(n_units + 3) / 4, 256, 0, st>>>(
+            (const XT *)x, (const XT *)gw, partial, (half_t *)x16, s->T, s->H, s->E, p.S, p.EG, n_units);
 }
 
 int odsd_launch_router(const odsd_moe_shape *s, const void *x, const void *gate_w, int32_t *idx, float *w,
@@ -279,8 +325,8 @@ int odsd_launch_router(const odsd_moe_shape *s, const void *x, const void *gate_
     else ROUTER_GO(1);
 #undef ROUTER_GO
     ODSD_CHECK_LAUNCH();
-    router_topk_kernel<<<(s->T + 3) / 4, 256, 0, st>>>(partial, s->T, s->E, s->K, p.S, s->renorm, idx, w,
-                                                        idx64);
+    router_topk_kernel<<<(s->T + 3) / 4, 256, 0, st>>>(partial, s->T, s->E, s->K,
+                                                        p.S % 4 == 0 ? p.S / 4 : p.S, s->renorm, idx, w, idx64);
     ODSD_CHECK_LAUNCH();
     return ODSD_OK;
 }
