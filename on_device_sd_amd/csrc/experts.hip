@@ -260,6 +260,8 @@ __global__ __launch_bounds__(256, OCC) void w4_gemm_kernel(const GemmParams p) {
         for (int g = g_begin; g < g_end;) {
 #pragma unroll
             for (int d = 0; d < DEPTH; ++d) {
+                // issue order is pinned: the DMA of the token rows two groups ahead first, then
+                // this slot's refill as soon as its codes have been expanded, then the products
                 const int xb = it % 3;
                 if (!DIRECT) dma_x((it + 2) % 3, g + 2);
                 __builtin_amdgcn_sched_barrier(0);
@@ -422,16 +424,14 @@ struct ExpertsPlan {
     int NB;          // 16-row weight blocks per wavefront
     int WK_gu, WK_dn;  // wavefronts splitting K inside a workgroup (MB == 1 path)
     int KS;          // split of the down projection's reduction dimension across workgroups
-    int variant;     // tuning knob (environment ODSD_GEMM_VARIANT), 0 = default
     size_t h_bytes, y_bytes;
 };
 
 // Choices are functions of the shape only (the per-expert counts live on the device).
 static ExpertsPlan experts_plan(const odsd_moe_shape *s) {
     ExpertsPlan p;
-    static const int env_variant = getenv("ODSD_GEMM_VARIANT") ? atoi(getenv("ODSD_GEMM_VARIANT")) : 0;
+    // tuning overrides for experiments: ODSD_GEMM_NB (2 or 4), ODSD_GEMM_KS (down-projection splits)
     static const int env_nb = getenv("ODSD_GEMM_NB") ? atoi(getenv("ODSD_GEMM_NB")) : 0;
-    p.variant = env_variant;
     const long P = (long)s->T * s->K;
     const long mean_rows = (P + s->E - 1) / s->E;
     if (s->T <= 16) p.MB = 1;
@@ -463,6 +463,8 @@ static ExpertsPlan experts_plan(const odsd_moe_shape *s) {
         while (KS * 2 <= G_dn / 2 && active * nchunks_dn * KS < 4 * slots && KS < 16) KS *= 2;
         p.KS = KS;
     }
+    static const int env_ks = getenv("ODSD_GEMM_KS") ? atoi(getenv("ODSD_GEMM_KS")) : 0;
+    if (env_ks > 0 && env_ks <= G_dn) p.KS = env_ks;
     // every split must own at least one group
     while (p.KS > 1 && ((G_dn + p.KS - 1) / p.KS) * (p.KS - 1) >= G_dn) p.KS--;
     p.h_bytes = odsd_round_up((size_t)(P > 0 ? P : 1) * s->I * sizeof(half_t), 256);
@@ -504,13 +506,8 @@ static void launch_gemm_plan(const ExpertsPlan &pl, GemmParams &gp, hipStream_t 
         if (pl.NB == 2) launch_gemm<2, 2, MODE, 3, 2, 1, false, 3>(gp, st);
         else launch_gemm<4, 2, MODE, 3, 4, 1, false, 2>(gp, st);
     } else if (pl.MB == 4) {
-        if (pl.NB == 2) {
-            if (pl.variant == 1) launch_gemm<2, 4, MODE, 3, 2, 1, false, 2>(gp, st);
-            else if (pl.variant == 2) launch_gemm<2, 4, MODE, 3, 2, 1, false, 3>(gp, st);
-            else launch_gemm<2, 4, MODE, 2, 2, 1, false, 3>(gp, st);
-        } else {
-            launch_gemm<4, 4, MODE, 2, 2, 1, false, 2>(gp, st);
-        }
+        if (pl.NB == 2) launch_gemm<2, 4, MODE, 2, 2, 1, false, 3>(gp, st);
+        else launch_gemm<4, 4, MODE, 2, 2, 1, false, 2>(gp, st);
     } else {
         launch_gemm<4, 8, MODE, 2, 4, 1, false, 1>(gp, st);
     }

@@ -90,7 +90,11 @@ class LayerInputs:
             # popularity rank of each expert: a seeded permutation, so that the hot experts
             # are spread over the id range
             rank = torch.randperm(wl.E, generator=self.g, device=self.device).to(torch.float32) + 1.0
-            bias = -wl.zipf_s * torch.log(rank)                      # log-popularity
+            # log-popularity, scaled to the spread of the unbiased logits (0.02*sqrt(H)): with
+            # Gaussian logit noise a factor of 0.5 makes the realised popularity fall off as
+            # rank^-s (log-log slope -1.1 for s = 1.1, ~100 of 128 experts hit by 64 tokens,
+            # as 8-of-128 sampling without replacement from Zipf(1.1) gives)
+            bias = -wl.zipf_s * torch.log(rank) * (ZIPF_BIAS_FACTOR * 0.02 * math.sqrt(wl.H))
             v = torch.full((wl.H,), 1.0 / math.sqrt(wl.H), device=self.device)
             wg = wg + (bias / ZIPF_SHIFT)[:, None] * v[None, :]
         return wg.to(wl.act_dtype)
@@ -116,3 +120,4 @@ class LayerInputs:
 
 # length of the activation component along the router's bias direction (Zipf configuration)
 ZIPF_SHIFT = 8.0
+ZIPF_BIAS_FACTOR = 0.5
