@@ -24,6 +24,14 @@ HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 HEADLINE = "mixtral_t160"
 
+# HBM bytes per launch of the gate_up kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
+# runs of this command (summaries and calibration in profiles/w4_gemm_gate_up_hbm_traffic.md):
+# FETCH_SIZE reads half of the bytes a plain 1 GiB device copy moves (factor 2.0), WRITE_SIZE
+# reads them in KiB (factor 1.0).
+MEASURED_TRAFFIC_BYTES = {
+    "mixtral_t160": 260742.9 * 2.0 * 1024 + 8961.2 * 1024,
+}
+
 
 def _build_layer(wl, dev, layer=0):
     import torch
@@ -110,7 +118,9 @@ def bench_layer(wl, dev, steps, warmup, with_cpu):
     else:
         ach = gu_bytes / (k_gu[0] * 1e-3) / 1e9
         roof = {"bound": "hbm", "kernel": "w4_gemm_kernel<gate_up>", "achieved": round(ach, 1),
-                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None}
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4),
+                "traffic": MEASURED_TRAFFIC_BYTES.get(wl.name)}
+        roof["algorithmic_bytes"] = gu_bytes
     roof["kernel_ms"] = round(k_gu[0], 4)
     layer_bytes_alg = wl.algorithmic_bytes(active)
     res = {
