@@ -20,92 +20,9 @@
 // Replaces: expert_forward_with_weights (demo/src/layers/mlp.py:227-230) inside the
 // per-expert loop of _execute_moe_with_placement (demo/src/model/qwen3_runner.py:303-380),
 // and the indexed "+=" combine (:363, :376).
-#include "common.h"
+#include "w4_gemm.h"
 
-
-typedef __attribute__((address_space(1))) uint4_t global_u4;
-typedef __attribute__((address_space(1))) uint32_t global_u32;
-typedef __attribute__((address_space(1))) char global_char;
-
-struct GemmParams {
-    const uint64_t *table;   // [E][4]
-    const half_t *src;       // activations, fp16
-    const int32_t *rowmap;   // slot -> source row (gate_up: token), or null: row = slot
-    const int32_t *counts;
-    const int32_t *offsets;
-    half_t *h16;             // MODE 0 output [P][I]
-    float *y;                // MODE 1 output [KS][P][ldo]
-    int src_ld;              // elements per source row (= reduction length Kd)
-    int G;                   // groups of 128 in the reduction dimension
-    int NBLK;                // 16-row blocks of the (fused) weight matrix
-    int nchunks;             // workgroup tiles along the rows
-    int KS;                  // splits of the reduction dimension
-    int gper;                // groups per split
-    int ldo;                 // I (MODE 0) or H (MODE 1)
-    int P;
-    int E;
-    int n_wg;                // E * nchunks * KS
-    int wg_per_xcd;          // ceil(n_wg / 8)
-};
-
-__device__ __forceinline__ half2_t as_half2(uint32_t u) { return __builtin_bit_cast(half2_t, u); }
-
-// Constants of the code -> fp16 bit trick.  (x & mask) | magic is one VOP3 instruction
-// (v_and_or_b32), but gfx9 VOP3 takes no literal and a single scalar operand, so with
-// compile-time constants the compiler emits v_and + v_or.  Passing the constants through an
-// empty asm once per kernel makes them opaque register values (masks in SGPRs, the magic
-// number in a VGPR), and the fused form is selected.
-struct DequantConsts {
-    uint32_t m_lo, m_hi, magic;
-};
-__device__ __forceinline__ DequantConsts dequant_consts() {
-    DequantConsts c{0x000F000Fu, 0x00F000F0u, 0x64006400u};
-    asm volatile("" : "+s"(c.m_lo), "+s"(c.m_hi), "+v"(c.magic));
-    return c;
-}
-
-// 4 words (32 codes) of one lane -> 4 x 8 fp16 weights  (w = (code - zero) * scale).
-// The integer part of the zero point is folded into the exact integer step that removes the
-// 1024 (low nibbles) / 64 (high nibbles, pre-scaled by 16) offset of the fp16 bit trick, so
-// only the fractional part of the zero point is rounded.
-__device__ __forceinline__ void dequant_tile(const DequantConsts &c, const uint4_t raw, const uint32_t szbits,
-                                             half8_t (&a)[4]) {
-    const half2_t sz = as_half2(szbits);
-    const half_t s = sz.x, z = sz.y;
-    const half_t zi = __builtin_rintf16(z);
-    const half_t zf = z - zi;                      // exact
-    const half_t c_lo = (half_t)(-1024.0f) - zi;   // exact for |zi| <= 1024
-    const half_t c_hi = (half_t)(-64.0f) - zi;
-    const half_t nz = -(zf * s);
-    const half2_t S = {s, s}, CLO = {c_lo, c_lo}, CHI = {c_hi, c_hi}, NZ = {nz, nz};
-    const half2_t R16 = {(half_t)0.0625f, (half_t)0.0625f};
-    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const uint32_t x = w[j], xs = x >> 8;
-        const half2_t t0 = as_half2((x & c.m_lo) | c.magic);
-        const half2_t t1 = as_half2((x & c.m_hi) | c.magic);
-        const half2_t t2 = as_half2((xs & c.m_lo) | c.magic);
-        const half2_t t3 = as_half2((xs & c.m_hi) | c.magic);
-        const half2_t q0 = t0 + CLO;
-        const half2_t q1 = __builtin_elementwise_fma(t1, R16, CHI);
-        const half2_t q2 = t2 + CLO;
-        const half2_t q3 = __builtin_elementwise_fma(t3, R16, CHI);
-        const half2_t v0 = __builtin_elementwise_fma(q0, S, NZ);
-        const half2_t v1 = __builtin_elementwise_fma(q1, S, NZ);
-        const half2_t v2 = __builtin_elementwise_fma(q2, S, NZ);
-        const half2_t v3 = __builtin_elementwise_fma(q3, S, NZ);
-        a[j] = half8_t{v0.x, v0.y, v1.x, v1.y, v2.x, v2.y, v3.x, v3.y};
-    }
-}
-
-__device__ __forceinline__ float silu_f32(float g) { return g / (1.0f + __expf(-g)); }
-
-// s_waitcnt vmcnt(N) only (gfx9 encoding: vmcnt = bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8)
-#define ODSD_WAIT_VMCNT(N) \
-    __builtin_amdgcn_s_waitcnt(((N) & 0xF) | (((N) >> 4) << 14) | (7 << 4) | (0xF << 8))
-
-typedef __attribute__((address_space(3))) void lds_void;
+#include <stdlib.h>
 
 // NB    16-row weight blocks per wavefront          MB  16-row token blocks per pass
 // DEPTH groups of weight loads kept in flight       NA  blocks expanded to fp16 at a time
@@ -117,25 +34,29 @@ typedef __attribute__((address_space(3))) void lds_void;
 //       (global_load_lds, no registers), three buffers deep, 16-byte segments XOR-swizzled
 //       by the row so that the B-fragment reads are bank-conflict free; one raw s_barrier
 //       per group, preceded by a vmcnt wait that leaves the newest loads in flight.
-template <int NB, int MB, int MODE, int DEPTH, int NA, int WK, bool DIRECT, int OCC>
-__global__ __launch_bounds__(256, OCC) void w4_gemm_kernel(const GemmParams p) {
+template <int NB, int MB, int MODE, int DEPTH, int NA, int WK, bool DIRECT, int OCC, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmParams p) {
     static_assert(MODE == 1 || NB % 2 == 0, "gate_up needs gate/up block pairs");
     static_assert(NB % NA == 0, "NA must divide NB");
     static_assert(!DIRECT || MB == 1, "the direct path holds one token block");
     static_assert(DIRECT || WK == 1, "K is split across wavefronts on the direct path only");
-    constexpr int RSUB = 4 / WK;                  // wavefronts along the rows
+    static_assert(!DIRECT || WAVES == 4, "the direct path uses 4 wavefronts");
+    static_assert((4 * MB) % WAVES == 0 || DIRECT, "token-row pieces must divide among the threads");
+    constexpr int RSUB = WAVES / WK;              // wavefronts along the rows
+    constexpr int XPT = DIRECT ? 1 : 4 * MB / WAVES;   // 16-byte pieces of a token-row chunk per thread
+    constexpr int ROWS_PER_PIECE = 4 * WAVES;     // rows covered by one piece index (16 threads per row)
     constexpr int XS_BYTES = DIRECT ? 16 : 3 * 16 * MB * 256;
     constexpr int RED_FLOATS = WK > 1 ? (WK - 1) * RSUB * 64 * NB * 4 : 1;
     __shared__ __attribute__((aligned(16))) char xs_raw[XS_BYTES];
     __shared__ __attribute__((aligned(16))) float red[RED_FLOATS];
 
     // workgroup -> (expert, row chunk, k split).  Hardware deals workgroups round-robin over
-    // the 8 XCDs.  With many token rows per expert (MB >= 8) consecutive logical ids are kept
+    // the 8 XCDs.  With many token rows per expert (MB >= 6) consecutive logical ids are kept
     // on one XCD so that an expert's rows stay in one L2; with few rows that locality is worth
     // nothing and would leave an XCD idle for every expert without tokens, so the chunks of
     // one expert are spread over all XCDs instead.
     const int b = blockIdx.x;
-    const int L = MB >= 8 ? (b & 7) * p.wg_per_xcd + (b >> 3) : b;
+    const int L = MB >= 6 ? (b & 7) * p.wg_per_xcd + (b >> 3) : b;
     if (L >= p.n_wg) return;
     const int ks = L % p.KS;
     const int chunk = (L / p.KS) % p.nchunks;
@@ -180,7 +101,7 @@ __global__ __launch_bounds__(256, OCC) void w4_gemm_kernel(const GemmParams p) {
         sz_off[i] = (blk * p.G * 16 + r) * 4u;
     }
 
-    // x staging (DMA path): piece = tid + 256 i -> row = piece / 16, segment = piece % 16
+    // x staging (DMA path): piece = tid + 64*WAVES*i -> row = piece / 16, segment = piece % 16
     const int st_seg = tid & 15;
     const int st_row0 = tid >> 4;
 
@@ -193,10 +114,10 @@ __global__ __launch_bounds__(256, OCC) void w4_gemm_kernel(const GemmParams p) {
         //   DIRECT path: row r of the block, columns 8*kq.. of each 32-column step
         // rows past the expert's last one are clamped to its first row: the MFMA columns they
         // feed are never stored
-        uint32_t st_off[MB];
+        uint32_t st_off[XPT];
 #pragma unroll
-        for (int i = 0; i < MB; ++i) {
-            const int row = DIRECT ? r : st_row0 + 16 * i;
+        for (int i = 0; i < XPT; ++i) {
+            const int row = DIRECT ? r : st_row0 + ROWS_PER_PIECE * i;
             const int slot = base + m0 + (row < mcnt ? row : 0);
             const int srow = p.rowmap ? p.rowmap[slot] : slot;
             const int seg = DIRECT ? kq : (st_seg ^ (row & 15));
@@ -229,12 +150,12 @@ __global__ __launch_bounds__(256, OCC) void w4_gemm_kernel(const GemmParams p) {
                 xd[DIRECT ? buf : 0][j] =
                     *(const global_u4 *)(src_c + (st_off[0] + gc * (ODSD_GROUP * 2u) + j * 64u));
         };
-        // MB asynchronous 16-byte loads per thread: global -> xs[buf] (no registers)
+        // XPT asynchronous 16-byte loads per thread: global -> xs[buf] (no registers)
         auto dma_x = [&](int buf, int g) {
             const uint32_t gc = (uint32_t)min(g, g_last);
 #pragma unroll
-            for (int i = 0; i < MB; ++i) {
-                lds_void *dst = (lds_void *)(xs_raw + buf * (16 * MB * 256) + (i * 256 + wave * 64) * 16);
+            for (int i = 0; i < XPT; ++i) {
+                lds_void *dst = (lds_void *)(xs_raw + buf * (16 * MB * 256) + (i * 64 * WAVES + wave * 64) * 16);
                 __builtin_amdgcn_global_load_lds((const global_u4 *)(src_c + (st_off[i] + gc * (ODSD_GROUP * 2u))),
                                                  dst, 16, 0, 0);
             }
@@ -252,7 +173,7 @@ __global__ __launch_bounds__(256, OCC) void w4_gemm_kernel(const GemmParams p) {
         }
         if (!DIRECT) {
             // x(g_begin) has landed once at most the loads issued after it are outstanding
-            ODSD_WAIT_VMCNT(MB + DEPTH * 2 * NB);
+            ODSD_WAIT_VMCNT(XPT + DEPTH * 2 * NB);
             __builtin_amdgcn_s_barrier();
         }
 
@@ -308,7 +229,7 @@ __global__ __launch_bounds__(256, OCC) void w4_gemm_kernel(const GemmParams p) {
                     __builtin_amdgcn_sched_barrier(0);
                     // x(g+1) was issued one step ago; the loads issued after it are that step's
                     // refill, this step's DMA and this step's refill
-                    ODSD_WAIT_VMCNT(4 * NB + MB);
+                    ODSD_WAIT_VMCNT(4 * NB + XPT);
                     __builtin_amdgcn_s_barrier();
                 }
                 ++g;
@@ -452,6 +373,8 @@ static ExpertsPlan experts_plan(const odsd_moe_shape *s) {
         p.KS = KS;
         const int gper = (G_dn + KS - 1) / KS;
         p.WK_dn = gper >= 8 ? 4 : (gper >= 4 ? 2 : 1);
+    } else if (p.MB >= 8) {
+        p.KS = 1;      // the prefill tile kernel reduces over the whole of I
     } else {
         if (p.MB <= 4) {
             const long wg_gu = active * ((2 * s->I / 16 + 15) / 16);
@@ -487,13 +410,16 @@ extern "C" size_t odsd_experts_workspace_bytes(const odsd_moe_shape *s) {
     return p.h_bytes + p.y_bytes;
 }
 
-template <int NB, int MB, int MODE, int DEPTH, int NA, int WK, bool DIRECT, int OCC>
+template <int NB, int MB, int MODE, int DEPTH, int NA, int WK, bool DIRECT, int OCC, int WAVES = 4>
 static void launch_gemm(GemmParams &gp, hipStream_t st) {
-    gp.nchunks = (gp.NBLK + (4 / WK) * NB - 1) / ((4 / WK) * NB);
+    gp.nchunks = (gp.NBLK + (WAVES / WK) * NB - 1) / ((WAVES / WK) * NB);
     gp.n_wg = gp.E * gp.nchunks * gp.KS;
     gp.wg_per_xcd = (gp.n_wg + 7) / 8;
-    w4_gemm_kernel<NB, MB, MODE, DEPTH, NA, WK, DIRECT, OCC><<<gp.wg_per_xcd * 8, 256, 0, st>>>(gp);
+    w4_gemm_kernel<NB, MB, MODE, DEPTH, NA, WK, DIRECT, OCC, WAVES><<<gp.wg_per_xcd * 8, 64 * WAVES, 0, st>>>(gp);
 }
+
+// prefill-shaped tile kernel (experts_prefill.hip)
+template <int MODE> void odsd_launch_gemm_prefill(GemmParams &gp, hipStream_t st);
 
 template <int MODE>
 static void launch_gemm_plan(const ExpertsPlan &pl, GemmParams &gp, hipStream_t st) {
@@ -509,7 +435,10 @@ static void launch_gemm_plan(const ExpertsPlan &pl, GemmParams &gp, hipStream_t 
         if (pl.NB == 2) launch_gemm<2, 4, MODE, 2, 2, 1, false, 3>(gp, st);
         else launch_gemm<4, 4, MODE, 2, 2, 1, false, 2>(gp, st);
     } else {
-        launch_gemm<4, 8, MODE, 2, 4, 1, false, 1>(gp, st);
+        // ODSD_GEMM_PREFILL=0 keeps the streaming kernel (for comparison runs)
+        static const int v = getenv("ODSD_GEMM_PREFILL") ? atoi(getenv("ODSD_GEMM_PREFILL")) : 1;
+        if (v == 1) odsd_launch_gemm_prefill<MODE>(gp, st);
+        else launch_gemm<4, 8, MODE, 2, 4, 1, false, 1>(gp, st);
     }
 }
 
