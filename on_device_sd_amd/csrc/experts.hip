@@ -156,8 +156,7 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
 #pragma unroll
             for (int i = 0; i < XPT; ++i) {
                 lds_void *dst = (lds_void *)(xs_raw + buf * (16 * MB * 256) + (i * 64 * WAVES + wave * 64) * 16);
-                __builtin_amdgcn_global_load_lds((const global_u4 *)(src_c + (st_off[i] + gc * (ODSD_GROUP * 2u))),
-                                                 dst, 16, 0, 0);
+                dma16_to_lds(src_c, st_off[i] + gc * (ODSD_GROUP * 2u), dst);
             }
         };
 
@@ -181,11 +180,11 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
         for (int g = g_begin; g < g_end;) {
 #pragma unroll
             for (int d = 0; d < DEPTH; ++d) {
-                // issue order is pinned: the DMA of the token rows two groups ahead first, then
-                // this slot's refill as soon as its codes have been expanded, then the products
+                // issue order is pinned: as soon as this slot's codes have been expanded, the DMA
+                // of the token rows two groups ahead and the slot's refill, then the products.
+                // (The compiler cannot see the DMA loads.  Issued after the expansion, the vmcnt
+                // wait it derives for the slot retires exactly the slot and the previous DMA.)
                 const int xb = it % 3;
-                if (!DIRECT) dma_x((it + 2) % 3, g + 2);
-                __builtin_amdgcn_sched_barrier(0);
                 half8_t bdir[4];
                 if (DIRECT) {
 #pragma unroll
@@ -199,6 +198,7 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
                     for (int i = 0; i < NA; ++i) dequant_tile(dc, wq[d][h + i], wsz[d][h + i], a[i]);
                     if (h + NA >= NB) {
                         __builtin_amdgcn_sched_barrier(0);
+                        if (!DIRECT) dma_x((it + 2) % 3, g + 2);
                         load_w(d, g + DEPTH);      // ring slot d is free again
                         __builtin_amdgcn_sched_barrier(0);
                     }
