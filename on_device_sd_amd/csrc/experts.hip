@@ -355,8 +355,10 @@ static ExpertsPlan experts_plan(const odsd_moe_shape *s) {
     static const int env_nb = getenv("ODSD_GEMM_NB") ? atoi(getenv("ODSD_GEMM_NB")) : 0;
     const long P = (long)s->T * s->K;
     const long mean_rows = (P + s->E - 1) / s->E;
+    // token blocks per pass follow the mean number of rows per expert; an expert with more
+    // rows than one pass holds takes further passes over its weights
     if (s->T <= 16) p.MB = 1;
-    else if (s->T <= 32) p.MB = 2;
+    else if (s->T <= 32 || mean_rows <= 16) p.MB = 2;
     else p.MB = (mean_rows * 3 / 2 <= 64) ? 4 : 8;
     const long active = s->E < P ? s->E : P;       // upper bound of experts with rows
     const long slots = 512;                        // 256 CUs x 2 workgroups
