@@ -43,6 +43,9 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
     static_assert(!DIRECT || WAVES == 4, "the direct path uses 4 wavefronts");
     static_assert((4 * MB) % WAVES == 0 || DIRECT, "token-row pieces must divide among the threads");
     constexpr int RSUB = WAVES / WK;              // wavefronts along the rows
+    // trips round the weight ring per loop iteration (the deeper rings serve short reductions,
+    // where a long unrolled body only costs instruction fetches)
+    constexpr int RING_TRIPS = DEPTH == 2 ? 4 : 1;
     constexpr int XPT = DIRECT ? 1 : 4 * MB / WAVES;   // 16-byte pieces of a token-row chunk per thread
     constexpr int ROWS_PER_PIECE = 4 * WAVES;     // rows covered by one piece index (16 threads per row)
     constexpr int XS_BYTES = DIRECT ? 16 : 3 * 16 * MB * 256;
@@ -178,8 +181,13 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
 
         int it = 0;
         for (int g = g_begin; g < g_end;) {
+            // The step loop is unrolled over several trips round the ring: at a loop header the
+            // compiler's wait-count bookkeeping falls back to draining every outstanding load
+            // before the first use of ring data, so the fewer headers the stream crosses, the
+            // less often the prefetch pipeline runs empty.
 #pragma unroll
-            for (int d = 0; d < DEPTH; ++d) {
+            for (int u = 0; u < DEPTH * RING_TRIPS; ++u) {
+                const int d = u % DEPTH;
                 // issue order is pinned: as soon as this slot's codes have been expanded, the DMA
                 // of the token rows two groups ahead and the slot's refill, then the products.
                 // (The compiler cannot see the DMA loads.  Issued after the expansion, the vmcnt

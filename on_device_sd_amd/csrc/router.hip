@@ -202,33 +202,51 @@ __global__ __launch_bounds__(256) void router_topk_kernel(const double *__restri
     double my_l = 0.0;
     double l_max = 0.0;
     for (int k = 0; k < K; ++k) {
-        // best remaining candidate of this lane: largest key, then lowest expert
+        // best remaining candidate of this lane: largest key, then lowest expert.  A lane with
+        // nothing left offers key 0 (no finite logit maps to it) and the largest expert id.
         uint64_t bk = 0;
         int be = 0x7fffffff;
-        double bl = 0.0;
 #pragma unroll
         for (int v = 0; v < ROUTER_MAX_V; ++v) {
             if (!((taken >> v) & 1u)) {
                 if (be == 0x7fffffff || key[v] > bk) {
                     bk = key[v];
                     be = lane + 64 * v;
-                    bl = lg[v];
                 }
             }
         }
+        // wavefront arg-max on (key, -expert) with DPP moves; the winner ends up in lane 63
+        uint32_t klo = (uint32_t)bk, khi = (uint32_t)(bk >> 32);
+#define ROUTER_DPP_STEP(CTRL, ROWMASK)                                                              \
+    {                                                                                               \
+        const uint32_t olo = (uint32_t)__builtin_amdgcn_update_dpp((int)klo, (int)klo, CTRL, ROWMASK, 0xF, false); \
+        const uint32_t ohi = (uint32_t)__builtin_amdgcn_update_dpp((int)khi, (int)khi, CTRL, ROWMASK, 0xF, false); \
+        const int oe = __builtin_amdgcn_update_dpp(be, be, CTRL, ROWMASK, 0xF, false);              \
+        const uint64_t ok = ((uint64_t)ohi << 32) | olo, mk = ((uint64_t)khi << 32) | klo;          \
+        const bool better = ok > mk || (ok == mk && oe < be);                                       \
+        klo = better ? olo : klo;                                                                   \
+        khi = better ? ohi : khi;                                                                   \
+        be = better ? oe : be;                                                                      \
+    }
+        ROUTER_DPP_STEP(0x111, 0xF)   // row_shr:1
+        ROUTER_DPP_STEP(0x112, 0xF)   // row_shr:2
+        ROUTER_DPP_STEP(0x114, 0xF)   // row_shr:4
+        ROUTER_DPP_STEP(0x118, 0xF)   // row_shr:8   -> lane 15 of every row holds the row's best
+        ROUTER_DPP_STEP(0x142, 0xA)   // row_bcast:15 into rows 1 and 3
+        ROUTER_DPP_STEP(0x143, 0xC)   // row_bcast:31 into rows 2 and 3 -> lane 63 holds the best
+#undef ROUTER_DPP_STEP
+        const int we = __builtin_amdgcn_readlane(be, 63);   // the same in every lane
+        // the winner's logit sits in lane (we & 63), slot (we >> 6)
+        double cand = lg[0];
 #pragma unroll
-        for (int o = 32; o > 0; o >>= 1) {
-            const uint64_t ok = __shfl_xor(bk, o, ODSD_WAVE);
-            const int oe = __shfl_xor(be, o, ODSD_WAVE);
-            const double ol = __shfl_xor(bl, o, ODSD_WAVE);
-            const bool better = (oe != 0x7fffffff) &&
-                                (be == 0x7fffffff || ok > bk || (ok == bk && oe < be));
-            if (better) { bk = ok; be = oe; bl = ol; }
-        }
-        // every lane now agrees on (be, bl)
-        if ((be & 63) == lane) taken |= 1u << (be >> 6);
-        if (lane == k) { my_e = be; my_l = bl; }
-        if (k == 0) l_max = bl;
+        for (int v = 1; v < ROUTER_MAX_V; ++v) cand = (we >> 6) == v ? lg[v] : cand;
+        const uint64_t cb = (uint64_t)__double_as_longlong(cand);
+        const uint32_t wlo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)cb, we & 63);
+        const uint32_t whi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(cb >> 32), we & 63);
+        const double wl = __longlong_as_double((long long)(((uint64_t)whi << 32) | wlo));
+        if ((we & 63) == lane) taken |= 1u << (we >> 6);
+        if (lane == k) { my_e = we; my_l = wl; }
+        if (k == 0) l_max = wl;
     }
 
     // weights in fp32; differences are taken in fp64 before the cast
