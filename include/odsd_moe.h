@@ -139,8 +139,10 @@ int odsd_experts_w4(const odsd_moe_shape *s, const void *x_f16, const uint64_t *
 
 /* The three kernels of odsd_experts_w4 one by one (same arguments, same results), for
  * callers that keep h / y themselves or time the stages:
- *   h_f16 fp16 [P, I] in slot order; y float [odsd_w4_down_splits(s)][P][H] partial sums
- *   over slices of I, which odsd_combine adds in slice order.
+ *   h_f16 fp16 [P, I] in slot order; y: a buffer of odsd_w4_down_splits(s)*P*H*4 bytes that
+ *   odsd_w4_down fills and odsd_combine reads -- float [splits][P][H] partial sums over slices
+ *   of I, which odsd_combine adds in slice order, or, at prefill shapes (splits == 1, more than
+ *   42 rows per expert on average), fp16 [P][H].
  * They stand in for the three F.linear calls of mlp.py:227-230 (gate/up fused with
  * SiLU*mul, then down) and the indexed "+=" of qwen3_runner.py:363. */
 int     odsd_w4_gate_up_silu(const odsd_moe_shape *s, const void *x_f16, const uint64_t *table,
@@ -148,8 +150,8 @@ int     odsd_w4_gate_up_silu(const odsd_moe_shape *s, const void *x_f16, const u
                              const int32_t *slot_token, void *h_f16, void *stream);
 int32_t odsd_w4_down_splits(const odsd_moe_shape *s);
 int     odsd_w4_down(const odsd_moe_shape *s, const void *h_f16, const uint64_t *table,
-                     const int32_t *counts, const int32_t *offsets, float *y, void *stream);
-int     odsd_combine(const odsd_moe_shape *s, const float *y, const int32_t *idx, const float *w,
+                     const int32_t *counts, const int32_t *offsets, void *y, void *stream);
+int     odsd_combine(const odsd_moe_shape *s, const void *y, const int32_t *idx, const float *w,
                      const int32_t *perm, const uint64_t *table, const void *residual,
                      float *out_f32, void *out_act, void *stream);
 

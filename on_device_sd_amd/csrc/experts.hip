@@ -305,7 +305,7 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
 // out_act = cast(residual + cast(moe)): the reference rounds the MoE output to the
 // activation dtype before the residual add (qwen3_runner.py:295, :226).
 // ---------------------------------------------------------------------------------------------
-template <typename XT>
+template <typename XT, bool YH>
 __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ y, const int32_t *__restrict__ idx,
                                                       const float *__restrict__ w,
                                                       const int32_t *__restrict__ perm,
@@ -322,8 +322,15 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
         const int slot = perm[pr];
         const int e = idx[pr];
         if (slot < 0 || e < 0 || e >= E || table[(size_t)e * ODSD_TABLE_COLS] == 0) continue;
-        float4_t v = *(const float4_t *)(y + (size_t)slot * H + c);
-        for (int s = 1; s < KS; ++s) v += *(const float4_t *)(y + ((size_t)s * P + slot) * H + c);
+        float4_t v;
+        if (YH) {
+            // prefill shapes: one fp16 value per output (KS == 1)
+            const half4_t hv = *(const half4_t *)((const half_t *)y + (size_t)slot * H + c);
+            v = float4_t{(float)hv.x, (float)hv.y, (float)hv.z, (float)hv.w};
+        } else {
+            v = *(const float4_t *)(y + (size_t)slot * H + c);
+            for (int s = 1; s < KS; ++s) v += *(const float4_t *)(y + ((size_t)s * P + slot) * H + c);
+        }
         const float wk = w[pr];
         acc.x = fmaf(wk, v.x, acc.x);
         acc.y = fmaf(wk, v.y, acc.y);
@@ -353,6 +360,7 @@ struct ExpertsPlan {
     int NB;          // 16-row weight blocks per wavefront
     int WK_gu, WK_dn;  // wavefronts splitting K inside a workgroup (MB == 1 path)
     int KS;          // split of the down projection's reduction dimension across workgroups
+    int y_f16;       // down-projection outputs kept as fp16 (prefill tile kernel) instead of fp32 partials
     size_t h_bytes, y_bytes;
 };
 
@@ -400,6 +408,10 @@ static ExpertsPlan experts_plan(const odsd_moe_shape *s) {
     if (env_ks > 0 && env_ks <= G_dn) p.KS = env_ks;
     // every split must own at least one group
     while (p.KS > 1 && ((G_dn + p.KS - 1) / p.KS) * (p.KS - 1) >= G_dn) p.KS--;
+    // At prefill shapes the fp32 partials would be 0.5 GB written and read back per layer; fp16
+    // still carries 3 more bits than the bf16 the reference keeps its expert outputs in.
+    static const int env_pf = getenv("ODSD_GEMM_PREFILL") ? atoi(getenv("ODSD_GEMM_PREFILL")) : 1;
+    p.y_f16 = p.MB >= 8 && env_pf == 1 && p.KS == 1;
     p.h_bytes = odsd_round_up((size_t)(P > 0 ? P : 1) * s->I * sizeof(half_t), 256);
     p.y_bytes = odsd_round_up((size_t)p.KS * (size_t)(P > 0 ? P : 1) * s->H * sizeof(float), 256);
     return p;
@@ -447,6 +459,7 @@ static void launch_gemm_plan(const ExpertsPlan &pl, GemmParams &gp, hipStream_t 
     } else {
         // ODSD_GEMM_PREFILL=0 keeps the streaming kernel (for comparison runs)
         static const int v = getenv("ODSD_GEMM_PREFILL") ? atoi(getenv("ODSD_GEMM_PREFILL")) : 1;
+        gp.y_f16 = pl.y_f16;
         if (v == 1) odsd_launch_gemm_prefill<MODE>(gp, st);
         else launch_gemm<4, 8, MODE, 2, 4, 1, false, 1>(gp, st);
     }
@@ -484,7 +497,7 @@ extern "C" int32_t odsd_w4_down_splits(const odsd_moe_shape *s) {
 
 // down: h_f16 [P,I] -> y [KS][P][H] fp32 partial sums over KS slices of I
 extern "C" int odsd_w4_down(const odsd_moe_shape *s, const void *h_f16, const uint64_t *table,
-                            const int32_t *counts, const int32_t *offsets, float *y, void *stream) {
+                            const int32_t *counts, const int32_t *offsets, void *y, void *stream) {
     const int rc = experts_args_ok(s);
     if (rc != ODSD_OK) return rc;
     if (s->T == 0) return ODSD_OK;
@@ -493,7 +506,7 @@ extern "C" int odsd_w4_down(const odsd_moe_shape *s, const void *h_f16, const ui
     const ExpertsPlan pl = experts_plan(s);
     GemmParams dn{};
     dn.table = table; dn.src = (const half_t *)h_f16; dn.rowmap = nullptr;
-    dn.counts = counts; dn.offsets = offsets; dn.h16 = nullptr; dn.y = y;
+    dn.counts = counts; dn.offsets = offsets; dn.h16 = nullptr; dn.y = (float *)y;
     dn.src_ld = s->I; dn.G = s->I / ODSD_GROUP; dn.NBLK = s->H / 16;
     dn.KS = pl.KS; dn.gper = (dn.G + pl.KS - 1) / pl.KS; dn.ldo = s->H; dn.P = s->T * s->K; dn.E = s->E;
     launch_gemm_plan<1>(pl, dn, (hipStream_t)stream);
@@ -502,12 +515,13 @@ extern "C" int odsd_w4_down(const odsd_moe_shape *s, const void *h_f16, const ui
 }
 
 // combine: y partials + routing weights (+ residual) -> out
-extern "C" int odsd_combine(const odsd_moe_shape *s, const float *y, const int32_t *idx, const float *w,
+extern "C" int odsd_combine(const odsd_moe_shape *s, const void *y_, const int32_t *idx, const float *w,
                             const int32_t *perm, const uint64_t *table, const void *residual,
                             float *out_f32, void *out_act, void *stream) {
     const int rc = experts_args_ok(s);
     if (rc != ODSD_OK) return rc;
     if (s->T == 0) return ODSD_OK;
+    const float *y = (const float *)y_;
     if (!y || !idx || !w || !perm || !table) return ODSD_ERR_NULL;
     if (!out_f32 && !out_act) return ODSD_ERR_NULL;
     if (!odsd_aligned16(y) || (out_f32 && !odsd_aligned16(out_f32))) return ODSD_ERR_ALIGN;
@@ -516,14 +530,17 @@ extern "C" int odsd_combine(const odsd_moe_shape *s, const float *y, const int32
     const int P = s->T * s->K;
     hipStream_t st = (hipStream_t)stream;
     const dim3 grid((s->H / 4 + 255) / 256, s->T);
-    if (s->act_dtype == ODSD_DT_BF16)
-        combine_kernel<uint16_t><<<grid, 256, 0, st>>>(y, idx, w, perm, table, (const uint16_t *)residual,
-                                                       out_f32, (uint16_t *)out_act, s->T, s->H, s->K,
-                                                       s->E, pl.KS, P);
-    else
-        combine_kernel<float><<<grid, 256, 0, st>>>(y, idx, w, perm, table, (const float *)residual,
-                                                    out_f32, (float *)out_act, s->T, s->H, s->K, s->E,
-                                                    pl.KS, P);
+#define COMBINE_GO(XT, YH)                                                                             \
+    combine_kernel<XT, YH><<<grid, 256, 0, st>>>(y, idx, w, perm, table, (const XT *)residual, out_f32, \
+                                                 (XT *)out_act, s->T, s->H, s->K, s->E, pl.KS, P)
+    if (s->act_dtype == ODSD_DT_BF16) {
+        if (pl.y_f16) COMBINE_GO(uint16_t, true);
+        else COMBINE_GO(uint16_t, false);
+    } else {
+        if (pl.y_f16) COMBINE_GO(float, true);
+        else COMBINE_GO(float, false);
+    }
+#undef COMBINE_GO
     ODSD_CHECK_LAUNCH();
     return ODSD_OK;
 }

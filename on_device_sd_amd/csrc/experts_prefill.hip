@@ -326,7 +326,13 @@ __global__ __launch_bounds__(512, 2) void w4_gemm_prefill_kernel(const GemmParam
                     for (int i = 0; i < 4; ++i) {
                         if (blk_ok[i]) {
                             const int n = (cblk0 + i) * 16 + kq * 4;
-                            *(float4_t *)(p.y + slot * p.ldo + n) = acc[i][m];
+                            if (p.y_f16) {
+                                const float4_t v = acc[i][m];
+                                *(half4_t *)((half_t *)p.y + slot * p.ldo + n) =
+                                    half4_t{f32_to_f16_sat(v.x), f32_to_f16_sat(v.y), f32_to_f16_sat(v.z), f32_to_f16_sat(v.w)};
+                            } else {
+                                *(float4_t *)(p.y + slot * p.ldo + n) = acc[i][m];
+                            }
                         }
                     }
                 }
