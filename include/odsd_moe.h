@@ -160,12 +160,17 @@ size_t odsd_moe_workspace_bytes(const odsd_moe_shape *s);
 /* router -> dispatch -> experts -> combine in one call, no host round trip.
  * norm_weight (optional): apply RMSNorm(x) first (x is then the residual stream and is
  * also used as `residual` when add_residual != 0).
- * Routing outputs out_idx/out_w/out_counts/out_offsets/out_perm are optional. */
+ * Routing outputs out_idx/out_w/out_counts/out_offsets/out_perm are optional.
+ * row_sumsq_out (optional, needs out_act): double [T][ceil(H/1024)], sums of squares of every
+ *   row of out_act, one per 1024-column chunk.
+ * row_sumsq_in  (optional): the same statistic of x, e.g. the previous block's row_sumsq_out;
+ *   with it and norm_weight the RMSNorm is folded into the router kernel (one launch fewer). */
 int odsd_moe_forward(const odsd_moe_shape *s, const void *x, const void *norm_weight,
                      float eps, const void *gate_w, const uint64_t *table,
                      int32_t add_residual, float *out_f32, void *out_act,
                      int32_t *out_idx, float *out_w, int32_t *out_counts,
                      int32_t *out_offsets, int32_t *out_perm,
+                     const double *row_sumsq_in, double *row_sumsq_out,
                      void *workspace, size_t workspace_bytes, void *stream);
 
 #ifdef __cplusplus

@@ -49,7 +49,7 @@ SIGNATURES = {
     "odsd_combine": (C.c_int, [_SP, _P, _P, _P, _P, _P, _P, _P, _P, _P]),
     "odsd_moe_workspace_bytes": (C.c_size_t, [_SP]),
     "odsd_moe_forward": (C.c_int, [_SP, _P, _P, C.c_float, _P, _P, C.c_int32, _P, _P, _P, _P, _P, _P,
-                                   _P, _P, C.c_size_t, _P]),
+                                   _P, _P, _P, _P, C.c_size_t, _P]),
 }
 
 _lib: Optional[C.CDLL] = None

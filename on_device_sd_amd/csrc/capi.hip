@@ -57,6 +57,7 @@ extern "C" int odsd_moe_forward(const odsd_moe_shape *s, const void *x, const vo
                                 const void *gate_w, const uint64_t *table, int32_t add_residual,
                                 float *out_f32, void *out_act, int32_t *out_idx, float *out_w,
                                 int32_t *out_counts, int32_t *out_offsets, int32_t *out_perm,
+                                const double *row_sumsq_in, double *row_sumsq_out,
                                 void *workspace, size_t workspace_bytes, void *stream) {
     if (!s) return ODSD_ERR_NULL;
     const size_t need = odsd_moe_workspace_bytes(s);
@@ -77,18 +78,22 @@ extern "C" int odsd_moe_forward(const odsd_moe_shape *s, const void *x, const vo
     int32_t *slot_token = (int32_t *)(ws + l.slot_token);
     void *x16 = ws + l.x16;
 
+    // RMSNorm: with the row statistics at hand (left by the previous block's combine) the router
+    // kernel normalises on the fly; otherwise the stand-alone kernel runs first
     const void *xin = x;
-    if (norm_weight) {
+    const bool fold = norm_weight && row_sumsq_in;
+    if (row_sumsq_out && !out_act) return ODSD_ERR_NULL;
+    if (norm_weight && !fold) {
         const int rc = odsd_rmsnorm(x, norm_weight, s->act_dtype, s->T, s->H, eps, ws + l.xn, stream);
         if (rc != ODSD_OK) return rc;
         xin = ws + l.xn;
     }
     int rc = odsd_launch_router(s, xin, gate_w, idx, w, nullptr, x16, ws + l.router,
-                                l.xn - l.router, st);
+                                l.xn - l.router, st, fold ? row_sumsq_in : nullptr, norm_weight, eps);
     if (rc != ODSD_OK) return rc;
     rc = odsd_launch_dispatch(s, idx, counts, offsets, perm, inv, slot_token, st);
     if (rc != ODSD_OK) return rc;
     return odsd_launch_experts(s, x16, table, idx, w, counts, offsets, perm, slot_token,
                                add_residual ? x : nullptr, out_f32, out_act, ws + l.experts,
-                               l.total - l.experts, st);
+                               l.total - l.experts, st, row_sumsq_out);
 }

@@ -89,9 +89,11 @@ static inline bool odsd_aligned16(const void *p) { return (((uintptr_t)p) & 15u)
 static inline size_t odsd_round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 // kernels implemented in the other translation units (host launchers)
+// norm_ss/norm_w/eps: when norm_ss is given, x is RMS-normalised on the fly from the per-row sums
+// of squares (the router and the fp16 copy then see RMSNorm(x))
 int odsd_launch_router(const odsd_moe_shape *s, const void *x, const void *gate_w, int32_t *idx,
                        float *w, int64_t *idx64, void *x16, void *ws, size_t ws_bytes,
-                       hipStream_t st);
+                       hipStream_t st, const double *norm_ss, const void *norm_w, float eps);
 int odsd_launch_dispatch(const odsd_moe_shape *s, const int32_t *idx, int32_t *counts,
                          int32_t *offsets, int32_t *perm, int32_t *inv, int32_t *slot_token,
                          hipStream_t st);
@@ -99,4 +101,4 @@ int odsd_launch_experts(const odsd_moe_shape *s, const void *x16, const uint64_t
                         const int32_t *idx, const float *w, const int32_t *counts,
                         const int32_t *offsets, const int32_t *perm, const int32_t *slot_token,
                         const void *residual, float *out_f32, void *out_act, void *ws,
-                        size_t ws_bytes, hipStream_t st);
+                        size_t ws_bytes, hipStream_t st, double *row_ss);

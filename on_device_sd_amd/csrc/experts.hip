@@ -305,52 +305,69 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
 // out_act = cast(residual + cast(moe)): the reference rounds the MoE output to the
 // activation dtype before the residual add (qwen3_runner.py:295, :226).
 // ---------------------------------------------------------------------------------------------
-template <typename XT, bool YH>
+template <typename XT, bool YH, bool STATS>
 __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ y, const int32_t *__restrict__ idx,
                                                       const float *__restrict__ w,
                                                       const int32_t *__restrict__ perm,
                                                       const uint64_t *__restrict__ table,
                                                       const XT *__restrict__ residual,
                                                       float *__restrict__ out_f32, XT *__restrict__ out_act,
+                                                      double *__restrict__ row_ss,
                                                       int T, int H, int K, int E, int KS, int P) {
+    // One workgroup per (token, 1024-column chunk).  STATS: it also leaves the sum of squares of
+    // what it stored in out_act, row_ss[t][chunk] -- the statistic the next block's RMSNorm
+    // starts from (chunk sums are added in ascending order by whoever consumes them).
     const int t = blockIdx.y;
-    const int c = (blockIdx.x * 256 + threadIdx.x) * 4;
-    if (c >= H) return;
-    float4_t acc = {0.f, 0.f, 0.f, 0.f};
-    for (int k = 0; k < K; ++k) {
-        const int pr = t * K + k;
-        const int slot = perm[pr];
-        const int e = idx[pr];
-        if (slot < 0 || e < 0 || e >= E || table[(size_t)e * ODSD_TABLE_COLS] == 0) continue;
-        float4_t v;
-        if (YH) {
-            // prefill shapes: one fp16 value per output (KS == 1)
-            const half4_t hv = *(const half4_t *)((const half_t *)y + (size_t)slot * H + c);
-            v = float4_t{(float)hv.x, (float)hv.y, (float)hv.z, (float)hv.w};
-        } else {
-            v = *(const float4_t *)(y + (size_t)slot * H + c);
-            for (int s = 1; s < KS; ++s) v += *(const float4_t *)(y + ((size_t)s * P + slot) * H + c);
+    double ss = 0.0;
+    {
+        const int c = (blockIdx.x * 256 + threadIdx.x) * 4;
+        if (c < H) {
+        float4_t acc = {0.f, 0.f, 0.f, 0.f};
+        for (int k = 0; k < K; ++k) {
+            const int pr = t * K + k;
+            const int slot = perm[pr];
+            const int e = idx[pr];
+            if (slot < 0 || e < 0 || e >= E || table[(size_t)e * ODSD_TABLE_COLS] == 0) continue;
+            float4_t v;
+            if (YH) {
+                // prefill shapes: one fp16 value per output (KS == 1)
+                const half4_t hv = *(const half4_t *)((const half_t *)y + (size_t)slot * H + c);
+                v = float4_t{(float)hv.x, (float)hv.y, (float)hv.z, (float)hv.w};
+            } else {
+                v = *(const float4_t *)(y + (size_t)slot * H + c);
+                for (int s = 1; s < KS; ++s) v += *(const float4_t *)(y + ((size_t)s * P + slot) * H + c);
+            }
+            const float wk = w[pr];
+            acc.x = fmaf(wk, v.x, acc.x);
+            acc.y = fmaf(wk, v.y, acc.y);
+            acc.z = fmaf(wk, v.z, acc.z);
+            acc.w = fmaf(wk, v.w, acc.w);
         }
-        const float wk = w[pr];
-        acc.x = fmaf(wk, v.x, acc.x);
-        acc.y = fmaf(wk, v.y, acc.y);
-        acc.z = fmaf(wk, v.z, acc.z);
-        acc.w = fmaf(wk, v.w, acc.w);
-    }
-    const size_t o = (size_t)t * H + c;
-    float res[4] = {0.f, 0.f, 0.f, 0.f};
-    if (residual) {
+        const size_t o = (size_t)t * H + c;
+        float res[4] = {0.f, 0.f, 0.f, 0.f};
+        if (residual) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) res[i] = ActIO<XT>::load(residual, o + i);
-    }
-    const float a[4] = {acc.x, acc.y, acc.z, acc.w};
-    if (out_f32) *(float4_t *)(out_f32 + o) = float4_t{a[0] + res[0], a[1] + res[1], a[2] + res[2], a[3] + res[3]};
-    if (out_act) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const float m = ActIO<XT>::round(a[i]);
-            ActIO<XT>::store(out_act, o + i, residual ? __fadd_rn(res[i], m) : m);
+            for (int i = 0; i < 4; ++i) res[i] = ActIO<XT>::load(residual, o + i);
         }
+        const float a[4] = {acc.x, acc.y, acc.z, acc.w};
+        if (out_f32) *(float4_t *)(out_f32 + o) = float4_t{a[0] + res[0], a[1] + res[1], a[2] + res[2], a[3] + res[3]};
+        if (out_act) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float m = ActIO<XT>::round(a[i]);
+                const float stored = ActIO<XT>::round(residual ? __fadd_rn(res[i], m) : m);
+                ActIO<XT>::store(out_act, o + i, stored);
+                if (STATS) ss += (double)stored * (double)stored;
+            }
+        }
+        }
+    }
+    if (STATS) {
+        __shared__ double red[4];
+        ss = wave_sum(ss);
+        if (lane_id() == 0) red[threadIdx.x >> 6] = ss;
+        __syncthreads();
+        if (threadIdx.x == 0) row_ss[(size_t)t * gridDim.x + blockIdx.x] = (red[0] + red[1]) + (red[2] + red[3]);
     }
 }
 
@@ -514,41 +531,54 @@ extern "C" int odsd_w4_down(const odsd_moe_shape *s, const void *h_f16, const ui
     return ODSD_OK;
 }
 
-// combine: y partials + routing weights (+ residual) -> out
-extern "C" int odsd_combine(const odsd_moe_shape *s, const void *y_, const int32_t *idx, const float *w,
-                            const int32_t *perm, const uint64_t *table, const void *residual,
-                            float *out_f32, void *out_act, void *stream) {
+// combine: y partials + routing weights (+ residual) -> out (+ per-row sum of squares of out_act)
+static int launch_combine(const odsd_moe_shape *s, const void *y_, const int32_t *idx, const float *w,
+                          const int32_t *perm, const uint64_t *table, const void *residual,
+                          float *out_f32, void *out_act, double *row_ss, hipStream_t st) {
     const int rc = experts_args_ok(s);
     if (rc != ODSD_OK) return rc;
     if (s->T == 0) return ODSD_OK;
     const float *y = (const float *)y_;
     if (!y || !idx || !w || !perm || !table) return ODSD_ERR_NULL;
     if (!out_f32 && !out_act) return ODSD_ERR_NULL;
+    if (row_ss && !out_act) return ODSD_ERR_NULL;
     if (!odsd_aligned16(y) || (out_f32 && !odsd_aligned16(out_f32))) return ODSD_ERR_ALIGN;
     if (s->T > 65535) return ODSD_ERR_UNSUPPORTED;
     const ExpertsPlan pl = experts_plan(s);
     const int P = s->T * s->K;
-    hipStream_t st = (hipStream_t)stream;
     const dim3 grid((s->H / 4 + 255) / 256, s->T);
-#define COMBINE_GO(XT, YH)                                                                             \
-    combine_kernel<XT, YH><<<grid, 256, 0, st>>>(y, idx, w, perm, table, (const XT *)residual, out_f32, \
-                                                 (XT *)out_act, s->T, s->H, s->K, s->E, pl.KS, P)
+#define COMBINE_GO(XT, YH, ST)                                                                          \
+    combine_kernel<XT, YH, ST><<<grid, 256, 0, st>>>(y, idx, w, perm, table, (const XT *)residual,     \
+                                                     out_f32, (XT *)out_act, row_ss, s->T, s->H, s->K, \
+                                                     s->E, pl.KS, P)
+#define COMBINE_Y(XT, ST)                          \
+    do {                                           \
+        if (pl.y_f16) COMBINE_GO(XT, true, ST);    \
+        else COMBINE_GO(XT, false, ST);            \
+    } while (0)
     if (s->act_dtype == ODSD_DT_BF16) {
-        if (pl.y_f16) COMBINE_GO(uint16_t, true);
-        else COMBINE_GO(uint16_t, false);
+        if (row_ss) COMBINE_Y(uint16_t, true);
+        else COMBINE_Y(uint16_t, false);
     } else {
-        if (pl.y_f16) COMBINE_GO(float, true);
-        else COMBINE_GO(float, false);
+        if (row_ss) COMBINE_Y(float, true);
+        else COMBINE_Y(float, false);
     }
+#undef COMBINE_Y
 #undef COMBINE_GO
     ODSD_CHECK_LAUNCH();
     return ODSD_OK;
 }
 
+extern "C" int odsd_combine(const odsd_moe_shape *s, const void *y, const int32_t *idx, const float *w,
+                            const int32_t *perm, const uint64_t *table, const void *residual,
+                            float *out_f32, void *out_act, void *stream) {
+    return launch_combine(s, y, idx, w, perm, table, residual, out_f32, out_act, nullptr, (hipStream_t)stream);
+}
+
 int odsd_launch_experts(const odsd_moe_shape *s, const void *x16, const uint64_t *table, const int32_t *idx,
                         const float *w, const int32_t *counts, const int32_t *offsets, const int32_t *perm,
                         const int32_t *slot_token, const void *residual, float *out_f32, void *out_act,
-                        void *ws, size_t ws_bytes, hipStream_t st) {
+                        void *ws, size_t ws_bytes, hipStream_t st, double *row_ss) {
     int rc = experts_check(s);
     if (rc != ODSD_OK) return rc;
     if (s->T == 0) return ODSD_OK;
@@ -562,7 +592,7 @@ int odsd_launch_experts(const odsd_moe_shape *s, const void *x16, const uint64_t
     if (rc != ODSD_OK) return rc;
     rc = odsd_w4_down(s, h16, table, counts, offsets, y, st);
     if (rc != ODSD_OK) return rc;
-    return odsd_combine(s, y, idx, w, perm, table, residual, out_f32, out_act, st);
+    return launch_combine(s, y, idx, w, perm, table, residual, out_f32, out_act, row_ss, st);
 }
 
 extern "C" int odsd_experts_w4(const odsd_moe_shape *s, const void *x_f16, const uint64_t *table,
@@ -571,5 +601,5 @@ extern "C" int odsd_experts_w4(const odsd_moe_shape *s, const void *x_f16, const
                                const void *residual, float *out_f32, void *out_act, void *workspace,
                                size_t workspace_bytes, void *stream) {
     return odsd_launch_experts(s, x_f16, table, idx, w, counts, offsets, perm, slot_token, residual,
-                               out_f32, out_act, workspace, workspace_bytes, (hipStream_t)stream);
+                               out_f32, out_act, workspace, workspace_bytes, (hipStream_t)stream, nullptr);
 }

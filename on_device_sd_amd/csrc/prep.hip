@@ -103,17 +103,28 @@ __global__ __launch_bounds__(256) void w4_pack_kernel(const uint8_t *__restrict_
 template <typename XT>
 __global__ __launch_bounds__(256) void rmsnorm_kernel(const XT *__restrict__ x, const XT *__restrict__ wt,
                                                       int H, double eps, XT *__restrict__ out) {
-    __shared__ double red[4];
+    __shared__ double red[2][4];
     const size_t row = (size_t)blockIdx.x * H;
-    double ss = 0.0;
-    for (int h = threadIdx.x; h < H; h += 256) {
-        const double v = (double)ActIO<XT>::load(x, row + h);
-        ss += v * v;
+    // The sum of squares is built exactly as the combine kernel builds the row statistic it
+    // leaves for the next block (per 1024-column chunk: 4 consecutive columns per thread, a
+    // wavefront sum, the 4 wavefront sums pairwise; chunks added in ascending order), so that
+    // the stand-alone and the folded RMSNorm give the same bits.
+    double tot = 0.0;
+    for (int c0 = 0, n = 0; c0 < H; c0 += 1024, ++n) {
+        const int c = c0 + (int)threadIdx.x * 4;
+        double ss = 0.0;
+        if (c < H) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const double v = (double)ActIO<XT>::load(x, row + c + i);
+                ss += v * v;
+            }
+        }
+        ss = wave_sum(ss);
+        if (lane_id() == 0) red[n & 1][threadIdx.x >> 6] = ss;
+        __syncthreads();
+        tot += (red[n & 1][0] + red[n & 1][1]) + (red[n & 1][2] + red[n & 1][3]);
     }
-    ss = wave_sum(ss);
-    if (lane_id() == 0) red[threadIdx.x >> 6] = ss;
-    __syncthreads();
-    const double tot = (red[0] + red[1]) + (red[2] + red[3]);
     const double r = 1.0 / sqrt(tot / (double)H + eps);
     for (int h = threadIdx.x; h < H; h += 256) {
         const float xn = ActIO<XT>::round((float)((double)ActIO<XT>::load(x, row + h) * r));

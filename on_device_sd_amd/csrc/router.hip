@@ -45,7 +45,9 @@ __global__ __launch_bounds__(256) void router_partial_kernel(const XT *__restric
                                                              const XT *__restrict__ wg,
                                                              double *__restrict__ partial,
                                                              half_t *__restrict__ x16, int T, int H,
-                                                             int E, int S, int EG, int n_units) {
+                                                             int E, int S, int EG, int n_units,
+                                                             const double *__restrict__ norm_ss,
+                                                             const XT *__restrict__ norm_w, double eps) {
     const int unit = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (unit >= n_units) return;
     const int lane = lane_id();
@@ -75,6 +77,16 @@ __global__ __launch_bounds__(256) void router_partial_kernel(const XT *__restric
 #pragma unroll
     for (int i = 0; i < NE; ++i) acc[i] = double4_t{0.0, 0.0, 0.0, 0.0};
 
+    // fused RMSNorm (demo/src/layers/layernorm.py:21-27): the row statistic comes from the kernel
+    // that produced x; the arithmetic per element is that of the stand-alone RMSNorm kernel
+    const bool normed = norm_ss != nullptr;
+    double rstd = 1.0;
+    if (normed) {
+        const int nchunk = (H + 1023) / 1024;   // the statistic arrives as per-chunk sums
+        double tot = 0.0;
+        for (int c = 0; c < nchunk; ++c) tot += norm_ss[(size_t)(t_ok ? t : 0) * nchunk + c];
+        rstd = 1.0 / sqrt(tot / (double)H + eps);
+    }
     const XT *xrow = x + (size_t)(t_ok ? t : 0) * H;
     const XT *wrow[NE];
     bool e_ok[NE];
@@ -89,6 +101,15 @@ __global__ __launch_bounds__(256) void router_partial_kernel(const XT *__restric
         const int h = k0 + c + kg * 8;
         float xa[8];
         Row8<XT>::load(xrow + h, xa);
+        if (normed) {
+            float nw[8];
+            Row8<XT>::load(norm_w + h, nw);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float xn = ActIO<XT>::round((float)((double)xa[j] * rstd));
+                xa[j] = ActIO<XT>::round(__fmul_rn(xn, nw[j]));
+            }
+        }
         if (!t_ok) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) xa[j] = 0.0f;
@@ -310,22 +331,27 @@ extern "C" size_t odsd_router_workspace_bytes(const odsd_moe_shape *s) {
 
 template <typename XT, int NE>
 static void launch_partial(const RouterPlan &p, const odsd_moe_shape *s, const void *x, const void *gw,
-                           double *partial, void *x16, hipStream_t st) {
+                           double *partial, void *x16, hipStream_t st, const double *norm_ss,
+                           const void *norm_w, float eps) {
     const int n_units = p.TT * p.EG * p.S;
     if (p.S % 4 == 0)
         router_partial_kernel<XT, NE, true><<<n_units / 4, 256, 0, st>>>(
-            (const XT *)x, (const XT *)gw, partial, (half_t *)x16, s->T, s->H, s->E, p.S, p.EG, n_units);
+            (const XT *)x, (const XT *)gw, partial, (half_t *)x16, s->T, s->H, s->E, p.S, p.EG, n_units,
+            norm_ss, (const XT *)norm_w, (double)eps);
     else
         router_partial_kernel<XT, NE, false><<<(n_units + 3) / 4, 256, 0, st>>>(
-            (const XT *)x, (const XT *)gw, partial, (half_t *)x16, s->T, s->H, s->E, p.S, p.EG, n_units);
+            (const XT *)x, (const XT *)gw, partial, (half_t *)x16, s->T, s->H, s->E, p.S, p.EG, n_units,
+            norm_ss, (const XT *)norm_w, (double)eps);
 }
 
 int odsd_launch_router(const odsd_moe_shape *s, const void *x, const void *gate_w, int32_t *idx, float *w,
-                       int64_t *idx64, void *x16, void *ws, size_t ws_bytes, hipStream_t st) {
+                       int64_t *idx64, void *x16, void *ws, size_t ws_bytes, hipStream_t st,
+                       const double *norm_ss, const void *norm_w, float eps) {
     const int rc = router_check(s);
     if (rc != ODSD_OK) return rc;
     if (s->T == 0) return ODSD_OK;
     if (!x || !gate_w || !idx || !w || !ws) return ODSD_ERR_NULL;
+    if (norm_ss && (!norm_w || !odsd_aligned16(norm_w))) return norm_w ? ODSD_ERR_ALIGN : ODSD_ERR_NULL;
     if (!odsd_aligned16(x) || !odsd_aligned16(gate_w) || !odsd_aligned16(ws) ||
         (x16 && !odsd_aligned16(x16)))
         return ODSD_ERR_ALIGN;
@@ -335,8 +361,8 @@ int odsd_launch_router(const odsd_moe_shape *s, const void *x, const void *gate_
     const bool bf = s->act_dtype == ODSD_DT_BF16;
 #define ROUTER_GO(NEV)                                                                   \
     do {                                                                                 \
-        if (bf) launch_partial<uint16_t, NEV>(p, s, x, gate_w, partial, x16, st);        \
-        else launch_partial<float, NEV>(p, s, x, gate_w, partial, x16, st);              \
+        if (bf) launch_partial<uint16_t, NEV>(p, s, x, gate_w, partial, x16, st, norm_ss, norm_w, eps); \
+        else launch_partial<float, NEV>(p, s, x, gate_w, partial, x16, st, norm_ss, norm_w, eps);       \
     } while (0)
     if (p.NE == 4) ROUTER_GO(4);
     else if (p.NE == 2) ROUTER_GO(2);
@@ -353,5 +379,5 @@ extern "C" int odsd_router_topk(const odsd_moe_shape *s, const void *x, const vo
                                 int32_t *out_idx, float *out_w, int64_t *out_idx64, void *x_f16,
                                 void *workspace, size_t workspace_bytes, void *stream) {
     return odsd_launch_router(s, x, gate_w, out_idx, out_w, out_idx64, x_f16, workspace, workspace_bytes,
-                              (hipStream_t)stream);
+                              (hipStream_t)stream, nullptr, nullptr, 0.0f);
 }

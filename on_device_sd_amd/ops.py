@@ -210,6 +210,12 @@ def experts_w4(x_f16: torch.Tensor, table: torch.Tensor, idx: torch.Tensor, w: t
     return out32, outa
 
 
+def row_stats(T: int, H: int, device) -> torch.Tensor:
+    """Buffer for the per-row sums of squares that one block's combine leaves for the next
+    block's RMSNorm (one double per row and 1024-column chunk)."""
+    return torch.empty(T, (H + 1023) // 1024, dtype=torch.float64, device=device)
+
+
 @dataclass
 class MoeOutputs:
     out_f32: Optional[torch.Tensor]
@@ -246,13 +252,23 @@ class MoeForwardPlan:
 
     def run(self, x: torch.Tensor, gate_weight: torch.Tensor, table: torch.Tensor,
             norm_weight: Optional[torch.Tensor] = None, eps: float = 1e-6,
-            add_residual: bool = False, out_act: Optional[torch.Tensor] = None) -> MoeOutputs:
+            add_residual: bool = False, out_act: Optional[torch.Tensor] = None,
+            row_sumsq_in: Optional[torch.Tensor] = None,
+            row_sumsq_out: Optional[torch.Tensor] = None) -> MoeOutputs:
+        """``row_sumsq_out`` (float64 [T, ceil(H/1024)], see ``row_stats``) receives the sums of
+        squares of every row of out_act; fed back as ``row_sumsq_in`` of the next block it lets
+        that block fold its RMSNorm into the router kernel."""
         lib = _lib.load()
         oa = out_act if out_act is not None else self.out_act
+        for ss in (row_sumsq_in, row_sumsq_out):
+            if ss is not None and (ss.dtype != torch.float64 or not ss.is_contiguous()
+                                   or ss.numel() != self.shape.T * ((self.shape.H + 1023) // 1024)):
+                raise ValueError("row statistics must be contiguous float64 [T, ceil(H/1024)]")
         _lib.check(lib.odsd_moe_forward(
             C.byref(self.shape), x.data_ptr(), _ptr(norm_weight), eps, gate_weight.data_ptr(),
             table.data_ptr(), 1 if add_residual else 0, _ptr(self.out_f32), _ptr(oa), _ptr(self.idx),
-            _ptr(self.w), _ptr(self.counts), _ptr(self.offsets), _ptr(self.perm), self.ws.data_ptr(),
+            _ptr(self.w), _ptr(self.counts), _ptr(self.offsets), _ptr(self.perm),
+            _ptr(row_sumsq_in), _ptr(row_sumsq_out), self.ws.data_ptr(),
             self.ws.numel(), _stream()), "odsd_moe_forward")
         return MoeOutputs(self.out_f32, oa, self.idx, self.w, self.counts, self.offsets, self.perm)
 

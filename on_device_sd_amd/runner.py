@@ -192,12 +192,18 @@ class MoEOnlyStack:
                                        want_f32=False, want_act=False, want_routing=False)
         self.buf = [torch.empty(T, config.hidden_size, dtype=self.dtype, device=self.device)
                     for _ in range(2)]
+        # per-row sum of squares of each hidden-state buffer: every layer's combine leaves it for
+        # the next layer, whose RMSNorm is then folded into its router kernel (layer 0 runs the
+        # stand-alone RMSNorm kernel)
+        self.rowss = [ops.row_stats(T, config.hidden_size, self.device) for _ in range(2)]
         self.graph = None
 
     def _run_layers(self):
         for l in range(self.L):
             self.plan.run(self.buf[l & 1], self.gate[l], self.tables[l], self.norm[l],
-                          self.config.rms_norm_eps, add_residual=True, out_act=self.buf[(l + 1) & 1])
+                          self.config.rms_norm_eps, add_residual=True, out_act=self.buf[(l + 1) & 1],
+                          row_sumsq_in=self.rowss[l & 1] if l > 0 else None,
+                          row_sumsq_out=self.rowss[(l + 1) & 1] if l + 1 < self.L else None)
 
     def capture(self):
         """Record the stack into a HIP graph (all kernels, no memset nodes)."""

@@ -58,9 +58,9 @@ def test_argument_checks_need_no_gpu():
     assert lib.odsd_router_topk(C.byref(ok), (1 << 20) + 4, 1 << 20, 1 << 20, 1 << 20, None, None, 1 << 20, 1 << 30, None) == 4
     assert lib.odsd_dispatch(C.byref(ok), None, None, None, None, None, None, None) == 1
     assert lib.odsd_moe_forward(C.byref(bad_h), None, None, 1e-6, None, None, 0, None, None, None, None, None,
-                                None, None, None, 0, None) == 2
+                                None, None, None, None, None, 0, None) == 2
     assert lib.odsd_moe_forward(C.byref(ok), 1 << 20, None, 1e-6, 1 << 20, 1 << 20, 0, None, None, None, None,
-                                None, None, None, 1 << 20, 16, None) == 5
+                                None, None, None, None, None, 1 << 20, 16, None) == 5
     assert lib.odsd_w4_packed_q_bytes(32, 256) == 32 * 256 // 2
     assert lib.odsd_w4_packed_sz_bytes(32, 256) == 32 * 2 * 4
     assert lib.odsd_w4_packed_q_bytes(30, 256) == 0

@@ -180,3 +180,37 @@ def test_moe_forward_vs_oracle(dev, T, H, E, K, I, dtype):
     # determinism: a second run gives the same bits
     out2 = ops.moe_forward(x.to(dev), wg.to(dev), bank.table(), K, I, renorm=True)
     assert torch.equal(out2.out_f32, out.out_f32)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H", [128, 1280, 2048])
+def test_rmsnorm_folded_into_router_matches_standalone(dev, H):
+    """Two chained blocks: the first block's combine leaves per-row sums of squares, the second
+    block folds its RMSNorm into the router kernel with them.  The result must equal, bit for
+    bit, the run in which the second block runs the stand-alone RMSNorm kernel, and the
+    statistic must be the sum of squares of the rows that were stored."""
+    import on_device_sd_amd as odsd
+    from on_device_sd_amd import ops
+    T, E, K, I = 37, 8, 2, 256
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev)
+    gate = (0.02 * torch.randn(E, H, generator=g)).to(torch.bfloat16).to(dev)
+    norm = (1 + 0.1 * torch.randn(H, generator=g)).to(torch.bfloat16).to(dev)
+    bank = odsd.W4ExpertBank(E, H, I, dev)
+    for e in range(E):
+        bank.load_expert(e, 0.02 * torch.randn(I, H, generator=g), 0.02 * torch.randn(I, H, generator=g),
+                         0.02 * torch.randn(H, I, generator=g))
+    plan = ops.MoeForwardPlan(T, H, E, K, I, True, torch.bfloat16, dev)
+    ss = ops.row_stats(T, H, dev)
+    h1 = torch.empty_like(x)
+    plan.run(x, gate, bank.table(), norm, 1e-6, add_residual=True, out_act=h1, row_sumsq_out=ss)
+    want_ss = (h1.double() ** 2).sum(dim=1)
+    got_ss = ss.sum(dim=1)
+    assert torch.allclose(got_ss, want_ss, rtol=1e-12, atol=0)
+    a = torch.empty_like(x)
+    b = torch.empty_like(x)
+    ra = plan.run(h1, gate, bank.table(), norm, 1e-6, add_residual=True, out_act=a)
+    idx_a = ra.idx.clone()
+    rb = plan.run(h1, gate, bank.table(), norm, 1e-6, add_residual=True, out_act=b, row_sumsq_in=ss)
+    assert torch.equal(idx_a, rb.idx)
+    assert torch.equal(a, b)
