@@ -78,7 +78,9 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
 
     const DequantConsts dc = dequant_consts();
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63;
+    // LDS path: the wavefront index as a scalar (the LDS targets of the copies are per wavefront)
+    const int wave = DIRECT ? (tid >> 6) : __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, kq = lane >> 4;
     const int kpart = wave % WK, rsub = wave / WK;
     // K range of the workgroup, then of this wavefront
@@ -107,6 +109,11 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
     // x staging (DMA path): piece = tid + 64*WAVES*i -> row = piece / 16, segment = piece % 16
     const int st_seg = tid & 15;
     const int st_row0 = tid >> 4;
+    // LDS byte offset of this lane's B fragment of 32-column step j inside a token block:
+    // row r, logical segment 4j + kq, stored at segment ^ (row & 15)
+    uint32_t lds_frag[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) lds_frag[j] = (uint32_t)((r * 16 + ((4 * j + kq) ^ r)) * 16);
 
     for (int m0 = 0; m0 < M_e; m0 += 16 * MB) {
         const int mcnt = min(M_e - m0, 16 * MB);
@@ -137,12 +144,17 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
         uint32_t wsz[DEPTH][NB];
         uint4_t xd[DIRECT ? DEPTH : 1][4];   // DIRECT: B fragments travel with the ring slot
 
+        // LDS path: the group advances a scalar base and the per-lane offsets never change (the
+        // direct path measured faster with the group folded into the per-lane offset)
         auto load_w = [&](int buf, int g) {
             const uint32_t gc = (uint32_t)min(g, g_last);
+            const global_char *qg = DIRECT ? qp_c : scalar_base(qp_c + (size_t)gc * 1024u);
+            const global_char *sg = DIRECT ? szp_c : scalar_base(szp_c + (size_t)gc * 64u);
+            const uint32_t gq = DIRECT ? gc * 1024u : 0u, gs = DIRECT ? gc * 64u : 0u;
 #pragma unroll
             for (int i = 0; i < NB; ++i) {
-                wq[buf][i] = __builtin_nontemporal_load((const global_u4 *)(qp_c + (wq_off[i] + gc * 1024u)));
-                wsz[buf][i] = *(const global_u32 *)(szp_c + (sz_off[i] + gc * 64u));
+                wq[buf][i] = __builtin_nontemporal_load((const global_u4 *)(qg + (wq_off[i] + gq)));
+                wsz[buf][i] = *(const global_u32 *)(sg + (sz_off[i] + gs));
             }
         };
         // DIRECT: the B fragments of group g (refilled only after the products that read them)
@@ -156,10 +168,11 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
         // XPT asynchronous 16-byte loads per thread: global -> xs[buf] (no registers)
         auto dma_x = [&](int buf, int g) {
             const uint32_t gc = (uint32_t)min(g, g_last);
+            const global_char *xg = src_c + (size_t)gc * (ODSD_GROUP * 2u);
 #pragma unroll
             for (int i = 0; i < XPT; ++i) {
                 lds_void *dst = (lds_void *)(xs_raw + buf * (16 * MB * 256) + (i * 64 * WAVES + wave * 64) * 16);
-                dma16_to_lds(src_c, st_off[i] + gc * (ODSD_GROUP * 2u), dst);
+                dma16_to_lds(xg, st_off[i], dst);
             }
         };
 
@@ -198,7 +211,11 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
 #pragma unroll
                     for (int j = 0; j < 4; ++j) bdir[j] = __builtin_bit_cast(half8_t, xd[DIRECT ? d : 0][j]);
                 }
-                const char *xbase = xs_raw + xb * (16 * MB * 256);
+                // this step's token buffer: one add per 32-column step, the block is an immediate
+                const char *xfrag[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) xfrag[j] = xs_raw + (uint32_t)(xb * (16 * MB * 256)) + lds_frag[j];
+                const int nmb_s = DIRECT ? nmb : scalar_int(nmb);
 #pragma unroll
                 for (int h = 0; h < NB; h += NA) {
                     half8_t a[NA][4];
@@ -212,17 +229,12 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
                     }
 #pragma unroll
                     for (int m = 0; m < MB; ++m) {
-                        if (m < nmb) {
+                        if (m < nmb_s) {
 #pragma unroll
                             for (int j = 0; j < 4; ++j) {
                                 half8_t bx;
-                                if (DIRECT) {
-                                    bx = bdir[j];
-                                } else {
-                                    // row m*16 + r, logical segment 4j + kq, stored at segment ^ (row & 15)
-                                    const int seg = (4 * j + kq) ^ r;
-                                    bx = *(const half8_t *)(xbase + ((m * 16 + r) * 16 + seg) * 16);
-                                }
+                                if (DIRECT) bx = bdir[j];
+                                else bx = *(const half8_t *)(xfrag[j] + m * 4096);
 #pragma unroll
                                 for (int i = 0; i < NA; ++i)
                                     acc[h + i][m] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i][j], bx, acc[h + i][m], 0, 0, 0);

@@ -103,6 +103,21 @@ __device__ __forceinline__ float silu_f32(float g) { return g / (1.0f + __expf(-
 
 typedef __attribute__((address_space(3))) void lds_void;
 
+// A wavefront-uniform global address as an opaque scalar: the compiler keeps it in an SGPR pair
+// and uses it as the scalar base of a global load (saddr form) instead of folding the uniform
+// part into the per-lane offset with a vector add per load.
+__device__ __forceinline__ const global_char *scalar_base(const global_char *p) {
+    asm volatile("" : "+s"(p));
+    return p;
+}
+// The same for a loop-invariant integer that should be compared on the scalar unit inside a loop
+// (hoisted out of the loop, such a comparison comes back as a lane mask that is moved through a
+// vector register on every trip).
+__device__ __forceinline__ int scalar_int(int v) {
+    asm volatile("" : "+s"(v));
+    return v;
+}
+
 // Asynchronous 16-byte-per-lane copy global -> LDS (no registers): lane l of the wavefront
 // writes dst + 16*l.  `dst` must be the same for all lanes.  Written as inline assembly on
 // purpose: the compiler models the builtin form as an access that may touch both memories,
