@@ -31,7 +31,7 @@
 // DIRECT == true  (MB == 1): token rows are never staged; each wavefront reads its B
 //       fragments straight from L1/L2 as part of the ring slot -- no barrier in the loop.
 // DIRECT == false (WK == 1): token rows go global -> LDS by asynchronous DMA loads
-//       (global_load_lds, no registers), three buffers deep, 16-byte segments XOR-swizzled
+//       (global_load_lds, no registers), double buffered, 16-byte segments XOR-swizzled
 //       by the row so that the B-fragment reads are bank-conflict free; one raw s_barrier
 //       per group, preceded by a vmcnt wait that leaves the newest loads in flight.
 template <int NB, int MB, int MODE, int DEPTH, int NA, int WK, bool DIRECT, int OCC, int WAVES>
@@ -48,10 +48,12 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
     constexpr int RING_TRIPS = DEPTH == 2 ? 4 : 1;
     constexpr int XPT = DIRECT ? 1 : 4 * MB / WAVES;   // 16-byte pieces of a token-row chunk per thread
     constexpr int ROWS_PER_PIECE = 4 * WAVES;     // rows covered by one piece index (16 threads per row)
-    constexpr int XS_BYTES = DIRECT ? 16 : 3 * 16 * MB * 256;
+    constexpr int XS_BYTES = 2 * 16 * MB * 256;
     constexpr int RED_FLOATS = WK > 1 ? (WK - 1) * RSUB * 64 * NB * 4 : 1;
-    __shared__ __attribute__((aligned(16))) char xs_raw[XS_BYTES];
-    __shared__ __attribute__((aligned(16))) float red[RED_FLOATS];
+    // one LDS object: token-row buffers (LDS path) or the K-part reduction area (direct path)
+    constexpr int LDS_BYTES = DIRECT ? (WK > 1 ? RED_FLOATS * 4 : 16) : XS_BYTES;
+    __shared__ __attribute__((aligned(16))) char xs_raw[LDS_BYTES];
+    float *red = (float *)xs_raw;
 
     // workgroup -> (expert, row chunk, k split).  Hardware deals workgroups round-robin over
     // the 8 XCDs.  With many token rows per expert (MB >= 6) consecutive logical ids are kept
@@ -118,6 +120,7 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
     for (int m0 = 0; m0 < M_e; m0 += 16 * MB) {
         const int mcnt = min(M_e - m0, 16 * MB);
         const int nmb = (mcnt + 15) >> 4;
+        const int mcnt_s = DIRECT ? mcnt : scalar_int(mcnt);
 
         // byte offsets of the token rows this thread fetches
         //   DMA path:    piece i -> row st_row0 + 16 i, source segment st_seg ^ (row & 15)
@@ -171,15 +174,18 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
             const global_char *xg = src_c + (size_t)gc * (ODSD_GROUP * 2u);
 #pragma unroll
             for (int i = 0; i < XPT; ++i) {
-                lds_void *dst = (lds_void *)(xs_raw + buf * (16 * MB * 256) + (i * 64 * WAVES + wave * 64) * 16);
-                dma16_to_lds(xg, st_off[i], dst);
+                // piece i covers ROWS_PER_PIECE rows from row ROWS_PER_PIECE * i on: nothing to
+                // fetch for a token block without rows
+                if (i * ROWS_PER_PIECE < mcnt_s) {
+                    lds_void *dst = (lds_void *)(xs_raw + buf * (16 * MB * 256) + (i * 64 * WAVES + wave * 64) * 16);
+                    dma16_to_lds(xg, st_off[i], dst);
+                }
             }
         };
 
         if (!DIRECT) {
             __builtin_amdgcn_s_barrier();   // the previous pass is done with xs
             dma_x(0, g_begin);
-            dma_x(1, g_begin + 1);
         }
 #pragma unroll
         for (int d = 0; d < DEPTH; ++d) {
@@ -188,7 +194,7 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
         }
         if (!DIRECT) {
             // x(g_begin) has landed once at most the loads issued after it are outstanding
-            ODSD_WAIT_VMCNT(XPT + DEPTH * 2 * NB);
+            ODSD_WAIT_VMCNT(DEPTH * 2 * NB);
             __builtin_amdgcn_s_barrier();
         }
 
@@ -202,10 +208,11 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
             for (int u = 0; u < DEPTH * RING_TRIPS; ++u) {
                 const int d = u % DEPTH;
                 // issue order is pinned: as soon as this slot's codes have been expanded, the DMA
-                // of the token rows two groups ahead and the slot's refill, then the products.
+                // of the next group's token rows (into the buffer the previous step read; every
+                // wavefront has passed that step's barrier) and the slot's refill, then the products.
                 // (The compiler cannot see the DMA loads.  Issued after the expansion, the vmcnt
                 // wait it derives for the slot retires exactly the slot and the previous DMA.)
-                const int xb = it % 3;
+                const int xb = it & 1;
                 half8_t bdir[4];
                 if (DIRECT) {
 #pragma unroll
@@ -223,7 +230,7 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
                     for (int i = 0; i < NA; ++i) dequant_tile(dc, wq[d][h + i], wsz[d][h + i], a[i]);
                     if (h + NA >= NB) {
                         __builtin_amdgcn_sched_barrier(0);
-                        if (!DIRECT) dma_x((it + 2) % 3, g + 2);
+                        if (!DIRECT) dma_x((it + 1) & 1, g + 1);
                         load_w(d, g + DEPTH);      // ring slot d is free again
                         __builtin_amdgcn_sched_barrier(0);
                     }
@@ -247,9 +254,10 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
                     load_xd(d, g + DEPTH);
                 } else {
                     __builtin_amdgcn_sched_barrier(0);
-                    // x(g+1) was issued one step ago; the loads issued after it are that step's
-                    // refill, this step's DMA and this step's refill
-                    ODSD_WAIT_VMCNT(4 * NB + XPT);
+                    // x(g+1) was issued in this step, before this step's refill: once only the
+                    // refill is outstanding it has landed (and so has the previous step's refill,
+                    // which the next step starts with anyway)
+                    ODSD_WAIT_VMCNT(2 * NB);
                     __builtin_amdgcn_s_barrier();
                 }
                 ++g;
@@ -405,6 +413,8 @@ static ExpertsPlan experts_plan(const odsd_moe_shape *s) {
     if (s->T <= 16) p.MB = 1;
     else if (s->T <= 32 || mean_rows <= 16) p.MB = 2;
     else p.MB = (mean_rows * 3 / 2 <= 64) ? 4 : 8;
+    static const int env_mb = getenv("ODSD_GEMM_MB") ? atoi(getenv("ODSD_GEMM_MB")) : 0;
+    if (env_mb >= 1 && env_mb <= 4) p.MB = env_mb;
     const long active = s->E < P ? s->E : P;       // upper bound of experts with rows
     const long slots = 512;                        // 256 CUs x 2 workgroups
     const int G_gu = s->H / ODSD_GROUP, G_dn = s->I / ODSD_GROUP;
@@ -480,10 +490,10 @@ static void launch_gemm_plan(const ExpertsPlan &pl, GemmParams &gp, hipStream_t 
         else if (wk == 2) launch_gemm<4, 1, MODE, 3, 2, 2, true, 2>(gp, st);
         else launch_gemm<4, 1, MODE, 3, 2, 1, true, 2>(gp, st);
     } else if (pl.MB == 2) {
-        if (pl.NB == 2) launch_gemm<2, 2, MODE, 3, 2, 1, false, 3>(gp, st);
+        if (pl.NB == 2) launch_gemm<2, 2, MODE, 2, 2, 1, false, 4>(gp, st);
         else launch_gemm<4, 2, MODE, 3, 4, 1, false, 2>(gp, st);
     } else if (pl.MB == 4) {
-        if (pl.NB == 2) launch_gemm<2, 4, MODE, 2, 2, 1, false, 3>(gp, st);
+        if (pl.NB == 2) launch_gemm<2, 4, MODE, 2, 2, 1, false, 4>(gp, st);
         else launch_gemm<4, 4, MODE, 2, 2, 1, false, 2>(gp, st);
     } else {
         // ODSD_GEMM_PREFILL=0 keeps the streaming kernel (for comparison runs)
