@@ -88,6 +88,34 @@ class W4ExpertBank:
         self.load_canonical(e, *canon)
         return canon if keep_canonical else None
 
+    EXPERT_WEIGHT_NAME = "model.layers.{layer}.mlp.experts.{expert}.{proj}_proj.weight"
+
+    def load_layer_from_state(self, state, layer_idx: int, name_format: Optional[str] = None,
+                              experts: Optional[Iterable[int]] = None) -> int:
+        """Quantise-on-load: take one layer's expert weights out of ``state`` (a mapping from
+        checkpoint tensor names to tensors, e.g. an opened safetensors shard or a state dict),
+        quantise and pack them on the device, one expert at a time, so that no more than one
+        expert's fp weights are resident besides the packed bank.  Names follow the checkpoint
+        layout the reference loader reads (``demo/src/memory/parameter_loader.py:424-539``):
+        ``model.layers.{L}.mlp.experts.{e}.{gate,up,down}_proj.weight`` with shapes [I,H], [I,H],
+        [H,I].  Experts whose tensors are missing from ``state`` are left unloaded.
+        Returns the number of experts loaded."""
+        fmt = name_format or self.EXPERT_WEIGHT_NAME
+        todo = range(self.num_experts) if experts is None else experts
+        loaded = 0
+        for e in todo:
+            names = [fmt.format(layer=layer_idx, expert=e, proj=p) for p in ("gate", "up", "down")]
+            if not all(n in state for n in names):
+                continue
+            gate, up, down = (state[n] for n in names)
+            if tuple(gate.shape) != (self.inter, self.hidden) or tuple(up.shape) != (self.inter, self.hidden) \
+                    or tuple(down.shape) != (self.hidden, self.inter):
+                raise ValueError(f"layer {layer_idx} expert {e}: unexpected weight shapes "
+                                 f"{tuple(gate.shape)}, {tuple(up.shape)}, {tuple(down.shape)}")
+            self.load_expert(e, gate, up, down)
+            loaded += 1
+        return loaded
+
     # -- views -------------------------------------------------------------------------------
     def expert_ptrs(self, e: int) -> Tuple[int, int, int, int]:
         return (self.gu_q[e].data_ptr(), self.gu_sz[e].data_ptr(),

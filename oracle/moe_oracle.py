@@ -27,6 +27,7 @@ Reference lines restated (paths relative to the reference tree):
   forward_moe        demo/src/model/qwen3_runner.py:212-226, :269-385
   RMSNorm            demo/src/layers/layernorm.py:21-27
   stack wiring       demo/src/layers/decoder_layer.py:126-140
+  activations        demo/src/execution/model_runner_utils.py:13-41
   quantiser form     pre_exp/expert_skip_prediction/quant.py:85-108 (applied per
                      128-column group instead of per tensor, 4 bits)
 
@@ -50,6 +51,9 @@ tests/test_oracle_*.py):
         substitution, 2-D/3-D shapes (demo/tests/unit/test_engine_optimizations.py
         :608-750, test_forward_moe.py:17-92).
   rmsnorm            closed form including the cast-before-weight order.
+  layer_activations  the set of (k, e, token) triples equals the set of nonzeros of the
+        one-hot expansion of the index matrix (brute force), tokens ascending, every pair
+        of the input appears exactly once.
 No function is "parity unpinned".
 """
 from __future__ import annotations
@@ -258,6 +262,22 @@ def dispatch(indices: np.ndarray, num_experts: int):
     perm = np.full(p, -1, dtype=np.int32)
     perm[order[:nvalid]] = np.arange(nvalid, dtype=np.int32)
     return counts, offsets, perm, inv
+
+
+def layer_activations(indices: np.ndarray, weights: np.ndarray, num_experts: int):
+    """The loop of build_layer_activations (model_runner_utils.py:20-34) restated: for every
+    rank k and expert e, in that order, the ascending tokens t with indices[t, k] == e and
+    their weights[t, k]; (k, e) pairs nobody selected are left out.
+    Returns a list of (k, e, tokens int64, weights)."""
+    indices = np.asarray(indices)
+    weights = np.asarray(weights)
+    out = []
+    for k in range(indices.shape[1]):
+        for e in range(num_experts):
+            tok = np.nonzero(indices[:, k] == e)[0].astype(np.int64)
+            if tok.size:
+                out.append((k, e, tok, weights[tok, k]))
+    return out
 
 
 # ----------------------------------------------------------------------------

@@ -177,3 +177,85 @@ def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libodsd_moe.so")
     with pytest.raises(ImportError, match="no\\s+CPU or PyTorch fallback"):
         _lib.load()
+
+
+@pytest.mark.gpu
+def test_build_layer_activations_matches_reference_loop(runner, dev):
+    """Device-side activation bookkeeping against the restated E x K loop of the reference."""
+    import on_device_sd_amd as odsd
+    cfg = runner.get_config()
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(41, cfg.hidden_size, generator=g).to(cfg.get_dtype()).to(dev)
+    rr = runner.route_experts(0, x)
+    acts = odsd.build_layer_activations(rr, cfg.num_experts)
+    want = orc.layer_activations(rr.topk_indices.cpu().numpy(), rr.topk_scores.cpu().numpy(), cfg.num_experts)
+    assert acts.layer_idx == 0 and acts.routing_scores is rr.topk_scores
+    assert len(acts.activations) == len(want)
+    for a, (k, e, tok, ww) in zip(acts.activations, want):
+        assert a.top_k_rank == k and a.expert_id == odsd.ExpertID(0, e)
+        assert a.token_indices.dtype == torch.int64
+        assert np.array_equal(a.token_indices.cpu().numpy(), tok)
+        assert np.array_equal(a.scores.cpu().numpy(), ww)
+
+
+@pytest.mark.gpu
+def test_build_prefill_placement_uses_resident_experts(runner, dev):
+    """Shared set, cache, loader are asked in the reference's order; an expert none of them
+    holds is left out of the placement, and the executor then skips it."""
+    import on_device_sd_amd as odsd
+    cfg = runner.get_config()
+    bank = runner.banks[0]
+
+    class Loader:
+        def __init__(self): self.asked = []
+        def is_shared_expert(self, eid): return eid.expert_idx == 0
+        def get_shared_expert_params(self, eid): return bank.expert_params(eid.expert_idx)
+        def get_expert_params(self, eid, device=None):
+            self.asked.append(eid.expert_idx)
+            return None if eid.expert_idx == 2 else bank.expert_params(eid.expert_idx)
+
+    class Cache:
+        def is_cached(self, eid): return eid.expert_idx == 1
+        def get(self, eid): return bank.expert_params(eid.expert_idx)
+
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(64, cfg.hidden_size, generator=g).to(cfg.get_dtype()).to(dev)
+    rr = runner.route_experts(0, x)
+    loader = Loader()
+    pl = odsd.build_prefill_placement(rr, Cache(), loader)
+    act = {e.expert_idx for e in rr.activated_expert_ids}
+    assert set(pl.gpu_expert_params) == act - {2} and pl.cpu_expert_params == {}
+    assert 0 not in loader.asked and 1 not in loader.asked
+    assert pl.routing_result is rr
+    out = runner._execute_moe_with_placement(x, pl)
+    assert out.shape == x.shape and torch.isfinite(out.float()).all()
+
+
+@pytest.mark.gpu
+def test_quantise_on_load_from_checkpoint_names(dev):
+    """A layer's experts taken out of a name -> tensor mapping (checkpoint naming of the
+    reference loader) give the same packed bytes as loading them one by one; experts whose
+    tensors are absent stay unloaded and show up as table row 0."""
+    import on_device_sd_amd as odsd
+    Hh, Ii, Ee, layer = 256, 128, 3, 5
+    g = torch.Generator().manual_seed(9)
+    state, ws = {}, {}
+    for e in (0, 2):
+        ws[e] = (torch.randn(Ii, Hh, generator=g) * 0.02, torch.randn(Ii, Hh, generator=g) * 0.02,
+                 torch.randn(Hh, Ii, generator=g) * 0.02)
+        for proj, t in zip(("gate", "up", "down"), ws[e]):
+            state[f"model.layers.{layer}.mlp.experts.{e}.{proj}_proj.weight"] = t.to(torch.bfloat16)
+    a = odsd.W4ExpertBank(Ee, Hh, Ii, dev)
+    assert a.load_layer_from_state(state, layer) == 2
+    assert a.loaded == [True, False, True]
+    b = odsd.W4ExpertBank(Ee, Hh, Ii, dev)
+    for e in (0, 2):
+        b.load_expert(e, *[t.to(torch.bfloat16) for t in ws[e]])
+    for name in ("gu_q", "gu_sz", "dn_q", "dn_sz"):
+        assert torch.equal(getattr(a, name), getattr(b, name))
+    tab = a.table().cpu()
+    assert (tab[1] == 0).all() and (tab[0] != 0).all() and (tab[2] != 0).all()
+    bad = dict(state)
+    bad[f"model.layers.{layer}.mlp.experts.0.down_proj.weight"] = torch.zeros(Ii, Hh)
+    with pytest.raises(ValueError):
+        odsd.W4ExpertBank(Ee, Hh, Ii, dev).load_layer_from_state(bad, layer)

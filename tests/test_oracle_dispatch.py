@@ -45,3 +45,28 @@ def test_dispatch_matches_stable_argsort_and_out_of_range():
     assert counts.tolist() == [2, 0, 3, 1] and offsets.tolist() == [0, 2, 2, 5, 6]
     assert perm.tolist() == [0, 1, 5, -1, -1, 2, 3, 4]
     assert inv.tolist() == [0, 1, 5, 6, 7, 2, -1, -1]
+
+
+def test_layer_activations_cover_every_pair_once():
+    """Pins oracle.layer_activations against a brute-force one-hot expansion: the (rank, expert,
+    token) triples are exactly the nonzeros of onehot[t, k, e], ordered by rank then expert with
+    ascending tokens, and the weights are those of the pair."""
+    rng = np.random.default_rng(5)
+    T, K, E = 23, 3, 7
+    idx = rng.integers(0, E, size=(T, K))
+    w = rng.random((T, K)).astype(np.float32)
+    acts = orc.layer_activations(idx, w, E)
+    onehot = np.zeros((T, K, E), dtype=bool)
+    for t in range(T):
+        for k in range(K):
+            onehot[t, k, idx[t, k]] = True
+    seen = np.zeros((T, K), dtype=int)
+    last = (-1, -1)
+    for k, e, tok, ww in acts:
+        assert (k, e) > last
+        last = (k, e)
+        assert tok.size > 0 and np.all(np.diff(tok) > 0)
+        assert np.array_equal(tok, np.nonzero(onehot[:, k, e])[0])
+        assert np.array_equal(ww, w[tok, k])
+        seen[tok, k] += 1
+    assert np.all(seen == 1)
