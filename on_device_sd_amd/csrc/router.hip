@@ -19,10 +19,13 @@
 #define ROUTER_MAX_NE 4    // expert tiles (of 16) per wavefront
 #define ROUTER_MAX_V 8     // logits per lane in the top-k kernel -> E <= 512
 
+// 8 consecutive activations of one row: the raw load and the conversion are separate so that
+// the loads of the next chunk can be in flight while the current one is multiplied
 template <typename XT> struct Row8;
 template <> struct Row8<uint16_t> {  // 8 bf16 = 16 bytes
-    __device__ static __forceinline__ void load(const uint16_t *p, float (&v)[8]) {
-        const uint4_t u = *(const uint4_t *)p;
+    typedef uint4_t Raw;
+    __device__ static __forceinline__ Raw raw(const uint16_t *p) { return *(const uint4_t *)p; }
+    __device__ static __forceinline__ void cvt(const Raw &u, float (&v)[8]) {
         const uint32_t w[4] = {u.x, u.y, u.z, u.w};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -32,10 +35,13 @@ template <> struct Row8<uint16_t> {  // 8 bf16 = 16 bytes
     }
 };
 template <> struct Row8<float> {
-    __device__ static __forceinline__ void load(const float *p, float (&v)[8]) {
-        const float4_t a = *(const float4_t *)p, b = *(const float4_t *)(p + 4);
-        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
-        v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    struct Raw { float4_t a, b; };
+    __device__ static __forceinline__ Raw raw(const float *p) {
+        return Raw{*(const float4_t *)p, *(const float4_t *)(p + 4)};
+    }
+    __device__ static __forceinline__ void cvt(const Raw &u, float (&v)[8]) {
+        v[0] = u.a.x; v[1] = u.a.y; v[2] = u.a.z; v[3] = u.a.w;
+        v[4] = u.b.x; v[5] = u.b.y; v[6] = u.b.z; v[7] = u.b.w;
     }
 };
 
@@ -97,13 +103,27 @@ __global__ __launch_bounds__(256) void router_partial_kernel(const XT *__restric
         wrow[i] = wg + (size_t)(e_ok[i] ? e : 0) * H;
     }
 
-    for (int c = 0; c < Hs; c += 32) {
+    // One chunk = 32 columns.  The raw loads of chunk c+1 are issued before chunk c is
+    // converted and multiplied (two register sets used in turn), so that their latency hides
+    // under the 8*NE fp64 MFMAs of the current chunk.
+    typedef typename Row8<XT>::Raw Raw;
+    struct Chunk {
+        Raw x, n, w[NE];
+    };
+    auto fetch = [&](Chunk &ck, int c) {
+        const int h = k0 + min(c, Hs - 32) + kg * 8;    // past the end: reload the last chunk
+        ck.x = Row8<XT>::raw(xrow + h);
+        if (normed) ck.n = Row8<XT>::raw(norm_w + h);
+#pragma unroll
+        for (int i = 0; i < NE; ++i) ck.w[i] = Row8<XT>::raw(wrow[i] + h);
+    };
+    auto consume = [&](const Chunk &ck, int c) {
         const int h = k0 + c + kg * 8;
         float xa[8];
-        Row8<XT>::load(xrow + h, xa);
+        Row8<XT>::cvt(ck.x, xa);
         if (normed) {
             float nw[8];
-            Row8<XT>::load(norm_w + h, nw);
+            Row8<XT>::cvt(ck.n, nw);
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const float xn = ActIO<XT>::round((float)((double)xa[j] * rstd));
@@ -126,13 +146,22 @@ __global__ __launch_bounds__(256) void router_partial_kernel(const XT *__restric
 #pragma unroll
         for (int i = 0; i < NE; ++i) {
             float wa[8];
-            Row8<XT>::load(wrow[i] + h, wa);
+            Row8<XT>::cvt(ck.w[i], wa);
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const double wd = e_ok[i] ? (double)wa[j] : 0.0;
                 acc[i] = __builtin_amdgcn_mfma_f64_16x16x4f64(xd[j], wd, acc[i], 0, 0, 0);
             }
         }
+    };
+    Chunk ca, cb;
+    fetch(ca, 0);
+    for (int c = 0; c < Hs; c += 64) {
+        fetch(cb, c + 32);
+        consume(ca, c);
+        if (c + 32 >= Hs) break;
+        fetch(ca, c + 64);
+        consume(cb, c + 32);
     }
 
     // When the K slices come in fours, the 4 wavefronts of this workgroup hold 4 consecutive
