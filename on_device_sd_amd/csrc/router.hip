@@ -17,7 +17,7 @@
 #include "common.h"
 
 #define ROUTER_MAX_NE 4    // expert tiles (of 16) per wavefront
-#define ROUTER_MAX_V 8     // logits per lane in the top-k kernel -> E <= 512
+#define ROUTER_MAX_V 8     // most logits per lane in the top-k kernel -> E <= 512
 
 // 8 consecutive activations of one row: the raw load and the conversion are separate so that
 // the loads of the next chunk can be in flight while the current one is multiplied
@@ -213,6 +213,8 @@ __device__ __forceinline__ uint64_t order_key(double v) {
     return (b >> 63) ? ~b : (b | 0x8000000000000000ull);
 }
 
+// V = logits per lane (experts lane, lane + 64, ...): 1, 2, 4 or 8 for E <= 64, 128, 256, 512
+template <int V>
 __global__ __launch_bounds__(256) void router_topk_kernel(const double *__restrict__ partial, int T, int E,
                                                           int K, int S, int renorm,
                                                           int32_t *__restrict__ idx,
@@ -222,28 +224,29 @@ __global__ __launch_bounds__(256) void router_topk_kernel(const double *__restri
     if (t >= T) return;
     const int lane = lane_id();
 
-    double lg[ROUTER_MAX_V];
-    uint64_t key[ROUTER_MAX_V];
+    double lg[V];
+    uint64_t key[V];
     uint32_t taken = 0;   // bit v set: expert lane + 64 v already selected
     // partial sums in slice order; the loads of one slice batch are independent of each other
 #pragma unroll
-    for (int v = 0; v < ROUTER_MAX_V; ++v) lg[v] = 0.0;
-    for (int s0 = 0; s0 < S; s0 += 4) {
-        double part[4][ROUTER_MAX_V];
+    for (int v = 0; v < V; ++v) lg[v] = 0.0;
+    constexpr int SB = V <= 2 ? 8 : 4;   // slices loaded together
+    for (int s0 = 0; s0 < S; s0 += SB) {
+        double part[SB][V];
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
+        for (int u = 0; u < SB; ++u)
 #pragma unroll
-            for (int v = 0; v < ROUTER_MAX_V; ++v) {
+            for (int v = 0; v < V; ++v) {
                 const int e = lane + 64 * v;
                 part[u][v] = (e < E && s0 + u < S) ? partial[((size_t)(s0 + u) * T + t) * E + e] : 0.0;
             }
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
+        for (int u = 0; u < SB; ++u)
 #pragma unroll
-            for (int v = 0; v < ROUTER_MAX_V; ++v) lg[v] += part[u][v];
+            for (int v = 0; v < V; ++v) lg[v] += part[u][v];
     }
 #pragma unroll
-    for (int v = 0; v < ROUTER_MAX_V; ++v) {
+    for (int v = 0; v < V; ++v) {
         key[v] = order_key(lg[v]);
         if (lane + 64 * v >= E) taken |= 1u << v;
     }
@@ -257,7 +260,7 @@ __global__ __launch_bounds__(256) void router_topk_kernel(const double *__restri
         uint64_t bk = 0;
         int be = 0x7fffffff;
 #pragma unroll
-        for (int v = 0; v < ROUTER_MAX_V; ++v) {
+        for (int v = 0; v < V; ++v) {
             if (!((taken >> v) & 1u)) {
                 if (be == 0x7fffffff || key[v] > bk) {
                     bk = key[v];
@@ -289,7 +292,7 @@ __global__ __launch_bounds__(256) void router_topk_kernel(const double *__restri
         // the winner's logit sits in lane (we & 63), slot (we >> 6)
         double cand = lg[0];
 #pragma unroll
-        for (int v = 1; v < ROUTER_MAX_V; ++v) cand = (we >> 6) == v ? lg[v] : cand;
+        for (int v = 1; v < V; ++v) cand = (we >> 6) == v ? lg[v] : cand;
         const uint64_t cb = (uint64_t)__double_as_longlong(cand);
         const uint32_t wlo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)cb, we & 63);
         const uint32_t whi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(cb >> 32), we & 63);
@@ -308,7 +311,7 @@ __global__ __launch_bounds__(256) void router_topk_kernel(const double *__restri
     } else {
         float part = 0.0f;
 #pragma unroll
-        for (int v = 0; v < ROUTER_MAX_V; ++v)
+        for (int v = 0; v < V; ++v)
             if (lane + 64 * v < E) part += expf((float)(lg[v] - l_max));
         den = wave_sum(part);
     }
@@ -398,8 +401,15 @@ int odsd_launch_router(const odsd_moe_shape *s, const void *x, const void *gate_
     else ROUTER_GO(1);
 #undef ROUTER_GO
     ODSD_CHECK_LAUNCH();
-    router_topk_kernel<<<(s->T + 3) / 4, 256, 0, st>>>(partial, s->T, s->E, s->K,
-                                                        p.S % 4 == 0 ? p.S / 4 : p.S, s->renorm, idx, w, idx64);
+    const int S_out = p.S % 4 == 0 ? p.S / 4 : p.S;
+#define TOPK_GO(VV)                                                                                   \
+    router_topk_kernel<VV><<<(s->T + 3) / 4, 256, 0, st>>>(partial, s->T, s->E, s->K, S_out, s->renorm, \
+                                                            idx, w, idx64)
+    if (s->E <= 64) TOPK_GO(1);
+    else if (s->E <= 128) TOPK_GO(2);
+    else if (s->E <= 256) TOPK_GO(4);
+    else TOPK_GO(8);
+#undef TOPK_GO
     ODSD_CHECK_LAUNCH();
     return ODSD_OK;
 }
