@@ -12,6 +12,9 @@
 
 #define DISPATCH_MAX_WAVES 16
 
+// ITERS > 0: a wavefront's segment is at most 64 * ITERS pairs long and the ids are kept in
+// registers between the two passes; ITERS == 0: any length, the ids are read twice.
+template <int ITERS>
 __global__ void dispatch_kernel(const int32_t *__restrict__ idx, int P, int K, int E,
                                 int32_t *__restrict__ counts, int32_t *__restrict__ offsets,
                                 int32_t *__restrict__ perm, int32_t *__restrict__ inv,
@@ -28,11 +31,25 @@ __global__ void dispatch_kernel(const int32_t *__restrict__ idx, int P, int K, i
     const int p_end = min(P, p_begin + seg);
 
     int c_eq = 0, c_lt = 0;
-    for (int p0 = p_begin; p0 < p_end; p0 += 64) {
-        const int p = p0 + lane;
-        const int v = p < p_end ? idx[p] : -1;
-        c_eq += __popcll(__ballot(v == e));
-        c_lt += __popcll(__ballot(v >= 0 && v < e));
+    int vals[ITERS > 0 ? ITERS : 1];
+    if (ITERS > 0) {
+#pragma unroll
+        for (int i = 0; i < ITERS; ++i) {
+            const int p = p_begin + i * 64 + lane;
+            vals[i] = p < p_end ? idx[p] : -1;
+        }
+#pragma unroll
+        for (int i = 0; i < ITERS; ++i) {
+            c_eq += __popcll(__ballot(vals[i] == e));
+            c_lt += __popcll(__ballot(vals[i] >= 0 && vals[i] < e));
+        }
+    } else {
+        for (int p0 = p_begin; p0 < p_end; p0 += 64) {
+            const int p = p0 + lane;
+            const int v = p < p_end ? idx[p] : -1;
+            c_eq += __popcll(__ballot(v == e));
+            c_lt += __popcll(__ballot(v >= 0 && v < e));
+        }
     }
     if (lane == 0) { s_eq[wave] = c_eq; s_lt[wave] = c_lt; }
     __syncthreads();
@@ -48,9 +65,7 @@ __global__ void dispatch_kernel(const int32_t *__restrict__ idx, int P, int K, i
         if (e == E - 1) offsets[E] = total_lt + total_eq;
     }
     int run = total_lt + base;
-    for (int p0 = p_begin; p0 < p_end; p0 += 64) {
-        const int p = p0 + lane;
-        const int v = p < p_end ? idx[p] : -1;
+    auto place = [&](int p, int v) {
         const uint64_t m = __ballot(v == e);
         if (v == e) {
             const int slot = run + mask_rank(m);
@@ -61,6 +76,15 @@ __global__ void dispatch_kernel(const int32_t *__restrict__ idx, int P, int K, i
         // expert 0's workgroup also marks pairs whose id no expert will claim
         if (e == 0 && p < p_end && (v < 0 || v >= E)) perm[p] = -1;
         run += __popcll(m);
+    };
+    if (ITERS > 0) {
+#pragma unroll
+        for (int i = 0; i < ITERS; ++i) place(p_begin + i * 64 + lane, vals[i]);
+    } else {
+        for (int p0 = p_begin; p0 < p_end; p0 += 64) {
+            const int p = p0 + lane;
+            place(p, p < p_end ? idx[p] : -1);
+        }
     }
     // slots past the last valid pair (only when some ids are out of range) are marked unused
     if (e == E - 1) {
@@ -81,7 +105,15 @@ int odsd_launch_dispatch(const odsd_moe_shape *s, const int32_t *idx, int32_t *c
     if (s->T == 0) return ODSD_OK;
     const int P = s->T * s->K;
     const int threads = P <= 4096 ? 256 : 1024;
-    dispatch_kernel<<<s->E, threads, 0, st>>>(idx, P, s->K, s->E, counts, offsets, perm, inv, slot_token);
+    const int nwaves = threads / 64;
+    const int iters = (((P + nwaves - 1) / nwaves + 63) & ~63) / 64;   // 64-pair chunks per wavefront
+#define DISPATCH_GO(IT) \
+    dispatch_kernel<IT><<<s->E, threads, 0, st>>>(idx, P, s->K, s->E, counts, offsets, perm, inv, slot_token)
+    if (iters <= 2) DISPATCH_GO(2);
+    else if (iters <= 8) DISPATCH_GO(8);
+    else if (iters <= 32) DISPATCH_GO(32);
+    else DISPATCH_GO(0);
+#undef DISPATCH_GO
     ODSD_CHECK_LAUNCH();
     return ODSD_OK;
 }
