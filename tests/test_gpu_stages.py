@@ -158,6 +158,10 @@ EXPERT_CASES = [
     (70, 384, 4, 2, 640, torch.bfloat16),     # >16 rows per expert, ragged row blocks (I/16 = 40)
     (200, 256, 2, 2, 256, torch.bfloat16),    # 200 rows per expert: several passes
     (64, 2048, 128, 8, 768, torch.bfloat16),  # config 3 shape (uniform routing)
+    # prefill tile kernel (mean rows per expert > 42) at awkward sizes:
+    (700, 384, 3, 2, 384, torch.bfloat16),    # odd group count, 1.5 row chunks in down, 2 passes per expert
+    (300, 640, 2, 1, 128, torch.float32),     # top-1, a single group in down, 2.5 row chunks, fp32 activations
+    (100, 256, 2, 2, 128, torch.bfloat16),    # 100 rows per expert: one partial pass
 ]
 
 
