@@ -23,27 +23,6 @@
 // demo/src/model/qwen3_runner.py:303-380.
 #include "w4_gemm.h"
 
-// ablation switches for timing experiments (never defined in the shipped build)
-#ifdef PF_ABLATE_BARRIER
-#define PF_BARRIER() __builtin_amdgcn_sched_barrier(0)
-#else
-#define PF_BARRIER() __builtin_amdgcn_s_barrier()
-#endif
-#ifdef PF_ABLATE_VMWAIT
-#define PF_WAIT(N) __builtin_amdgcn_sched_barrier(0)
-#else
-#define PF_WAIT(N) ODSD_WAIT_VMCNT_LGKM0(N)
-#endif
-#ifdef PF_ABLATE_MFMA
-static __device__ __forceinline__ float4_t pf_sink(half8_t a, half8_t b, float4_t c) {
-    asm volatile("" ::"v"(a), "v"(b));
-    return c;
-}
-#define PF_MFMA(a, b, c) pf_sink((a), (b), (c))
-#else
-#define PF_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_f16((a), (b), (c), 0, 0, 0)
-#endif
-
 template <int MODE, int MBW>
 __global__ __launch_bounds__(512, 2) void w4_gemm_prefill_kernel(const GemmParams p) {
     constexpr int BM = 2 * 16 * MBW;           // token rows per pass
@@ -132,9 +111,6 @@ __global__ __launch_bounds__(512, 2) void w4_gemm_prefill_kernel(const GemmParam
             }
         };
         auto dma_x = [&](char *xs, int st) {
-#ifdef PF_ABLATE_DMA
-            if (st > 1) return;
-#endif
             const uint32_t sc = (uint32_t)min(st, NST - 1);
 #pragma unroll
             for (int i = 0; i < XPT; ++i) {
@@ -148,29 +124,18 @@ __global__ __launch_bounds__(512, 2) void w4_gemm_prefill_kernel(const GemmParam
         // expand the two 32-column steps `half` (0: words x,y  1: words z,w) of ring slot `slot`
         // into weight buffer `buf`
         auto expand = [&](int slot, int half, char *ws) {
-#ifdef PF_ABLATE_EXPAND
-            if (m0 >= 0) return;
-#endif
 #pragma unroll
             for (int i = 0; i < 2; ++i) {
                 const DequantPrep pr = dequant_prep(wsz[slot][i]);
                 const uint32_t w0 = half ? wq[slot][i].z : wq[slot][i].x;
                 const uint32_t w1 = half ? wq[slot][i].w : wq[slot][i].y;
                 char *dst = ws + (((2 * wave + i) * 2) * 64 + lane) * 16;
-#ifdef PF_ABLATE_DEQ
-                *(uint4_t *)dst = uint4_t{w0, w1, w0, w1};
-                *(uint4_t *)(dst + 1024) = uint4_t{w1, w0, w1, w0};
-#else
                 *(half8_t *)dst = dequant_word(dc, pr, w0);
                 *(half8_t *)(dst + 1024) = dequant_word(dc, pr, w1);
-#endif
             }
         };
         // one quarter of expand(): duty tile i, word w of the half
         auto expand_piece = [&](int slot, int half, char *ws, int i, int w) {
-#ifdef PF_ABLATE_EXPAND
-            if (m0 >= 0) return;
-#endif
             const DequantPrep pr = dequant_prep(wsz[slot][i]);
             const uint32_t word = half ? (w ? wq[slot][i].w : wq[slot][i].z) : (w ? wq[slot][i].y : wq[slot][i].x);
             char *dst = ws + (((2 * wave + i) * 2) * 64 + lane) * 16 + w * 1024;
@@ -216,7 +181,7 @@ __global__ __launch_bounds__(512, 2) void w4_gemm_prefill_kernel(const GemmParam
         if ((U) < 4) expand_piece(eslot, ehalf, ews, (U) >> 1, (U) & 1);                                \
         _Pragma("unroll") for (int q = 0; q < 2; ++q)                                                   \
         _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                   \
-            acc[i][2 * mp + q] = PF_MFMA(a_cur[i], b_cur[q], acc[i][2 * mp + q]);                       \
+            acc[i][2 * mp + q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_cur[i], b_cur[q], acc[i][2 * mp + q], 0, 0, 0);                       \
         __builtin_amdgcn_sched_barrier(0);                                                              \
         if ((U) + 1 < 2 * UPJ) {                                                                        \
             if (((U) + 1) % UPJ == 0) {                                                                 \
@@ -273,15 +238,15 @@ __global__ __launch_bounds__(512, 2) void w4_gemm_prefill_kernel(const GemmParam
             __builtin_amdgcn_sched_barrier(0);
             load_w(0, g + 2);                  // slot 0 is fully expanded
             __builtin_amdgcn_sched_barrier(0);
-            PF_WAIT(4);          // the DMA is older than the 4 refill loads
-            PF_BARRIER();
+            ODSD_WAIT_VMCNT_LGKM0(4);          // the DMA is older than the 4 refill loads
+            __builtin_amdgcn_s_barrier();
             // stage 4k+1 : group g, second half.  produce (g+1, first half) -> x buf 0, w buf 0
             dma_x(xs0, 2 * g + 2);
             __builtin_amdgcn_sched_barrier(0);
             mma_stage(xs1, ws1, 1, 0, ws0);
             __builtin_amdgcn_sched_barrier(0);
-            PF_WAIT(0);
-            PF_BARRIER();
+            ODSD_WAIT_VMCNT_LGKM0(0);
+            __builtin_amdgcn_s_barrier();
             if (g + 1 >= G) break;
             // stage 4k+2 : group g+1, first half.  produce (g+1, second half) -> buffers 1
             dma_x(xs1, 2 * g + 3);
@@ -290,15 +255,15 @@ __global__ __launch_bounds__(512, 2) void w4_gemm_prefill_kernel(const GemmParam
             __builtin_amdgcn_sched_barrier(0);
             load_w(1, g + 3);
             __builtin_amdgcn_sched_barrier(0);
-            PF_WAIT(4);
-            PF_BARRIER();
+            ODSD_WAIT_VMCNT_LGKM0(4);
+            __builtin_amdgcn_s_barrier();
             // stage 4k+3 : group g+1, second half.  produce (g+2, first half) -> buffers 0
             dma_x(xs0, 2 * g + 4);
             __builtin_amdgcn_sched_barrier(0);
             mma_stage(xs1, ws1, 0, 0, ws0);
             __builtin_amdgcn_sched_barrier(0);
-            PF_WAIT(0);
-            PF_BARRIER();
+            ODSD_WAIT_VMCNT_LGKM0(0);
+            __builtin_amdgcn_s_barrier();
         }
 
         // epilogue: lane holds rows 4*kq..4*kq+3 of each 16-row tile, token column r

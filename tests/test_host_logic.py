@@ -73,3 +73,36 @@ def test_cpu_tensors_are_refused():
         ops.router_topk(torch.zeros(4, 128), torch.zeros(8, 128), 2, True)
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         ops.w4_quantize(torch.zeros(16, 128))
+
+
+def test_prefill_placement_lookup_order_without_gpu():
+    """build_prefill_placement is host logic: shared set first, then the cache, then the loader;
+    experts nobody holds are left out; nothing is placed on the CPU."""
+    import torch
+    from on_device_sd_amd.core import ExpertID, RoutingResult
+    from on_device_sd_amd.placement import build_prefill_placement
+
+    calls = []
+
+    class Loader:
+        def is_shared_expert(self, eid):
+            calls.append(("shared?", eid.expert_idx))
+            return eid.expert_idx == 3
+        def get_shared_expert_params(self, eid):
+            return {"who": "shared"}
+        def get_expert_params(self, eid, device=None):
+            calls.append(("loader", eid.expert_idx))
+            return None if eid.expert_idx == 5 else {"who": "loader"}
+
+    class Cache:
+        def is_cached(self, eid):
+            return eid.expert_idx == 4
+        def get(self, eid):
+            return {"who": "cache"}
+
+    rr = RoutingResult(layer_idx=2, topk_indices=torch.zeros(1, 1, dtype=torch.int64),
+                       topk_scores=torch.ones(1, 1), activated_expert_ids={ExpertID(2, e) for e in (3, 4, 5, 6)})
+    pl = build_prefill_placement(rr, Cache(), Loader())
+    assert {e: p["who"] for e, p in pl.gpu_expert_params.items()} == {3: "shared", 4: "cache", 6: "loader"}
+    assert pl.cpu_expert_params == {} and pl.substitution_map == {} and pl.routing_result is rr
+    assert ("loader", 3) not in calls and ("loader", 4) not in calls and ("loader", 5) in calls
