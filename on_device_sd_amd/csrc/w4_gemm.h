@@ -132,6 +132,6 @@ __device__ __forceinline__ void dma16_to_lds(const global_char *base, uint32_t b
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :
                  : "s"(m0v), "v"(byte_off), "s"(base)
-                 : "memory");
+                 : "memory");   // m0 is a reserved register: the compiler sets it itself before every use
 }
 
