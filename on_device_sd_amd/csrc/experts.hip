@@ -440,7 +440,7 @@ static ExpertsPlan experts_plan(const odsd_moe_shape *s) {
         }
         const int nchunks_dn = (s->H / 16 + 4 * p.NB - 1) / (4 * p.NB);
         int KS = 1;
-        while (KS * 2 <= G_dn / 2 && active * nchunks_dn * KS < 4 * slots && KS < 16) KS *= 2;
+        while (KS * 2 <= G_dn / 2 && active * nchunks_dn * KS < 2 * slots && KS < 16) KS *= 2;
         p.KS = KS;
     }
     static const int env_ks = getenv("ODSD_GEMM_KS") ? atoi(getenv("ODSD_GEMM_KS")) : 0;
