@@ -426,7 +426,7 @@ static ExpertsPlan experts_plan(const odsd_moe_shape *s) {
         p.WK_gu = G_gu >= 8 ? 4 : (G_gu >= 4 ? 2 : 1);
         const long chunks_dn = (s->H / 16 + 4 - 1) / 4;   // with WK = 4: 64 rows per workgroup
         int KS = 1;
-        while (KS * 2 <= G_dn / 8 && active * chunks_dn * KS < 8 * slots && KS < 16) KS *= 2;
+        while (KS * 2 <= G_dn / 8 && active * chunks_dn * KS < 4 * slots && KS < 16) KS *= 2;
         p.KS = KS;
         const int gper = (G_dn + KS - 1) / KS;
         p.WK_dn = gper >= 8 ? 4 : (gper >= 4 ? 2 : 1);
