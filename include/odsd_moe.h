@@ -101,6 +101,13 @@ int odsd_w4_pack(const uint8_t *q, const uint16_t *scale, const uint16_t *zero,
 /* out = cast(x * rsqrt(mean(x^2) + eps)) * weight, cast BEFORE the weight multiply. */
 int odsd_rmsnorm(const void *x, const void *weight, int32_t dtype, int32_t T, int32_t H,
                  float eps, void *out, void *stream);
+/* Fused residual add + RMSNorm, RMSNorm.add_rms_forward of demo/src/layers/layernorm.py:29-36
+ * (the post-attention norm of a real decoder layer, qwen3_runner.py:201-204):
+ *   s = float(x) + float(residual); residual_out = cast(s);
+ *   out = cast(s * rsqrt(mean(s^2) + eps)) * weight   (statistics over the unrounded sum).
+ * out / residual_out may alias x / residual. */
+int odsd_add_rmsnorm(const void *x, const void *residual, const void *weight, int32_t dtype,
+                     int32_t T, int32_t H, float eps, void *out, void *residual_out, void *stream);
 
 /* ---- Router ------------------------------------------------------------------------- */
 size_t odsd_router_workspace_bytes(const odsd_moe_shape *s);

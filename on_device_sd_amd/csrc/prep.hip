@@ -132,6 +132,34 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const XT *__restrict__ x, 
     }
 }
 
+// Fused residual add + RMSNorm (RMSNorm.add_rms_forward, demo/src/layers/layernorm.py:29-36):
+//   s = float(x) + float(residual); residual_out = cast(s);
+//   normed = cast(s * rsqrt(mean(s^2) + eps)) * weight   -- statistics over the UNROUNDED sum s.
+// One workgroup per token; the sum is recomputed in the second sweep instead of being kept.
+template <typename XT>
+__global__ __launch_bounds__(256) void add_rmsnorm_kernel(const XT *__restrict__ x, const XT *__restrict__ res,
+                                                          const XT *__restrict__ wt, int H, double eps,
+                                                          XT *__restrict__ out, XT *__restrict__ res_out) {
+    __shared__ double red[4];
+    const size_t row = (size_t)blockIdx.x * H;
+    double ss = 0.0;
+    for (int h = threadIdx.x; h < H; h += 256) {
+        const float s = __fadd_rn(ActIO<XT>::load(x, row + h), ActIO<XT>::load(res, row + h));
+        ss += (double)s * (double)s;
+    }
+    ss = wave_sum(ss);
+    if (lane_id() == 0) red[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    const double tot = (red[0] + red[1]) + (red[2] + red[3]);
+    const double r = 1.0 / sqrt(tot / (double)H + eps);
+    for (int h = threadIdx.x; h < H; h += 256) {
+        const float s = __fadd_rn(ActIO<XT>::load(x, row + h), ActIO<XT>::load(res, row + h));
+        ActIO<XT>::store(res_out, row + h, s);
+        const float xn = ActIO<XT>::round((float)((double)s * r));
+        ActIO<XT>::store(out, row + h, __fmul_rn(xn, ActIO<XT>::load(wt, h)));
+    }
+}
+
 template <typename XT>
 __global__ __launch_bounds__(256) void convert_f16_kernel(const XT *__restrict__ x, int64_t n,
                                                           half_t *__restrict__ o) {
@@ -197,6 +225,26 @@ extern "C" int odsd_rmsnorm(const void *x, const void *weight, int32_t dtype, in
     else if (dtype == ODSD_DT_BF16)
         rmsnorm_kernel<uint16_t><<<T, 256, 0, st>>>((const uint16_t *)x, (const uint16_t *)weight, H,
                                                     (double)eps, (uint16_t *)out);
+    else
+        return ODSD_ERR_DTYPE;
+    ODSD_CHECK_LAUNCH();
+    return ODSD_OK;
+}
+
+extern "C" int odsd_add_rmsnorm(const void *x, const void *residual, const void *weight, int32_t dtype,
+                                int32_t T, int32_t H, float eps, void *out, void *residual_out, void *stream) {
+    if (!x || !residual || !weight || !out || !residual_out) return ODSD_ERR_NULL;
+    if (T < 0 || H <= 0) return ODSD_ERR_SHAPE;
+    if (T == 0) return ODSD_OK;
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == ODSD_DT_F32)
+        add_rmsnorm_kernel<float><<<T, 256, 0, st>>>((const float *)x, (const float *)residual,
+                                                     (const float *)weight, H, (double)eps, (float *)out,
+                                                     (float *)residual_out);
+    else if (dtype == ODSD_DT_BF16)
+        add_rmsnorm_kernel<uint16_t><<<T, 256, 0, st>>>((const uint16_t *)x, (const uint16_t *)residual,
+                                                        (const uint16_t *)weight, H, (double)eps,
+                                                        (uint16_t *)out, (uint16_t *)residual_out);
     else
         return ODSD_ERR_DTYPE;
     ODSD_CHECK_LAUNCH();

@@ -98,6 +98,24 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6) -> torch.T
     return out.view(x.shape)
 
 
+def add_rmsnorm(x: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor,
+                eps: float = 1e-6) -> Tuple[torch.Tensor, torch.Tensor]:
+    """RMSNorm.forward(x, residual) of the reference (layernorm.py:29-47): returns
+    (normed, new_residual) with new_residual = cast(x + residual)."""
+    _require_cuda(x, residual, weight)
+    if x.shape != residual.shape or x.dtype != residual.dtype:
+        raise ValueError("x and residual must have the same shape and dtype")
+    lib = _lib.load()
+    x2 = x.contiguous().view(-1, x.shape[-1])
+    r2 = residual.contiguous().view(-1, x.shape[-1])
+    out = torch.empty_like(x2)
+    res_out = torch.empty_like(x2)
+    _lib.check(lib.odsd_add_rmsnorm(x2.data_ptr(), r2.data_ptr(), weight.to(x.dtype).contiguous().data_ptr(),
+                                    _dtype_code(x.dtype), x2.shape[0], x2.shape[1], eps, out.data_ptr(),
+                                    res_out.data_ptr(), _stream()), "odsd_add_rmsnorm")
+    return out.view(x.shape), res_out.view(x.shape)
+
+
 def to_f16(x: torch.Tensor) -> torch.Tensor:
     _require_cuda(x)
     lib = _lib.load()

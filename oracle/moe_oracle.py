@@ -25,7 +25,7 @@ Reference lines restated (paths relative to the reference tree):
   expert SwiGLU      demo/src/layers/mlp.py:209-231
   combine            demo/src/model/qwen3_runner.py:295, :363, :376
   forward_moe        demo/src/model/qwen3_runner.py:212-226, :269-385
-  RMSNorm            demo/src/layers/layernorm.py:21-27
+  RMSNorm            demo/src/layers/layernorm.py:21-27, fused add form :29-36
   stack wiring       demo/src/layers/decoder_layer.py:126-140
   activations        demo/src/execution/model_runner_utils.py:13-41
   quantiser form     pre_exp/expert_skip_prediction/quant.py:85-108 (applied per
@@ -51,6 +51,9 @@ tests/test_oracle_*.py):
         substitution, 2-D/3-D shapes (demo/tests/unit/test_engine_optimizations.py
         :608-750, test_forward_moe.py:17-92).
   rmsnorm            closed form including the cast-before-weight order.
+  add_rmsnorm        closed form in numpy float64 on the fp32 sum; a case where taking the
+        statistics over the rounded residual instead of the unrounded sum changes the result;
+        residual = 0 reduces it to rmsnorm.
   layer_activations  the set of (k, e, token) triples equals the set of nonzeros of the
         one-hot expansion of the index matrix (brute force), tokens ascending, every pair
         of the input appears exactly once.
@@ -366,6 +369,18 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6) -> torch.T
     var = xd.pow(2).mean(dim=-1, keepdim=True)
     y = (xd * torch.rsqrt(var + eps)).to(torch.float32).to(x.dtype)
     return y * weight.to(x.dtype)
+
+
+def add_rmsnorm(x: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6):
+    """layernorm.py:29-36: s = x.float() + residual.float(); residual_out = s.to(dtype); the
+    statistics and the normalisation use the UNROUNDED fp32 sum s; cast, then the weight.
+    (Statistics in fp64, as in rmsnorm above.)  Returns (normed, residual_out)."""
+    s = x.to(torch.float32) + residual.to(torch.float32)
+    res_out = s.to(x.dtype)
+    sd = s.to(torch.float64)
+    var = sd.pow(2).mean(dim=-1, keepdim=True)
+    y = (sd * torch.rsqrt(var + eps)).to(torch.float32).to(x.dtype)
+    return y * weight.to(x.dtype), res_out
 
 
 def moe_block(x: torch.Tensor, gate_weight: torch.Tensor, experts, top_k: int, renorm: bool):

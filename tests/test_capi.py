@@ -53,6 +53,8 @@ def test_argument_checks_need_no_gpu():
     assert lib.odsd_w4_pack(None, None, None, 16, 128, 1, 0, None, None, None) == 1
     assert lib.odsd_w4_pack(1 << 20, 1 << 20, 1 << 20, 10, 128, 1, 0, 1 << 20, 1 << 20, None) == 2
     assert lib.odsd_rmsnorm(None, None, 1, 4, 128, 1e-6, None, None) == 1
+    assert lib.odsd_add_rmsnorm(None, None, None, 1, 4, 128, 1e-6, None, None, None) == 1
+    assert lib.odsd_add_rmsnorm(1 << 20, 1 << 20, 1 << 20, 7, 4, 128, 1e-6, 1 << 20, 1 << 20, None) == 7
     assert lib.odsd_router_topk(C.byref(ok), None, None, None, None, None, None, None, 0, None) == 1
     assert lib.odsd_router_topk(C.byref(ok), 1 << 20, 1 << 20, 1 << 20, 1 << 20, None, None, 1 << 20, 16, None) == 5
     assert lib.odsd_router_topk(C.byref(ok), (1 << 20) + 4, 1 << 20, 1 << 20, 1 << 20, None, None, 1 << 20, 1 << 30, None) == 4

@@ -218,3 +218,28 @@ def test_rmsnorm_folded_into_router_matches_standalone(dev, H):
     rb = plan.run(h1, gate, bank.table(), norm, 1e-6, add_residual=True, out_act=b, row_sumsq_in=ss)
     assert torch.equal(idx_a, rb.idx)
     assert torch.equal(a, b)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_add_rmsnorm(dev, dtype):
+    """Fused residual add + RMSNorm against the oracle: the new residual is bit-exact, the normed
+    output within one unit in the last place on a tiny fraction of the elements (fp64 statistics
+    summed in a different order)."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(21)
+    T, H = 37, 1280
+    x = (torch.randn(T, H, generator=g) * 2).to(dtype)
+    r = (torch.randn(T, H, generator=g) * 2).to(dtype)
+    w = (1 + 0.2 * torch.randn(H, generator=g)).to(dtype)
+    got, res = ops.add_rmsnorm(x.to(dev), r.to(dev), w.to(dev), 1e-6)
+    want, want_res = orc.add_rmsnorm(x, r, w, 1e-6)
+    assert torch.equal(res.cpu(), want_res)
+    if dtype == torch.bfloat16:
+        ulp = (got.cpu().view(torch.int16).int() - want.view(torch.int16).int()).abs()
+        assert ulp.max() <= 1 and (ulp > 0).float().mean() < 1e-3
+    else:
+        torch.testing.assert_close(got.cpu(), want, rtol=1e-6, atol=1e-7)
+    # 3-D input keeps its shape
+    got3, res3 = ops.add_rmsnorm(x.to(dev).view(1, T, H), r.to(dev).view(1, T, H), w.to(dev), 1e-6)
+    assert got3.shape == (1, T, H) and torch.equal(got3.view(T, H), got) and torch.equal(res3.view(T, H), res)

@@ -127,6 +127,30 @@ def test_rmsnorm_cast_before_weight():
     torch.testing.assert_close(orc.rmsnorm(x32, w32, 1e-6), ref32, rtol=1e-6, atol=1e-7)
 
 
+def test_add_rmsnorm_uses_the_unrounded_sum():
+    # layernorm.py:29-36: x = x.float() + residual.float(); residual = x.to(orig); var over x (fp32)
+    g = torch.Generator().manual_seed(12)
+    x = (torch.randn(32, 256, generator=g) * 2).to(torch.bfloat16)
+    r = (torch.randn(32, 256, generator=g) * 2).to(torch.bfloat16)
+    w = (1 + 0.3 * torch.randn(256, generator=g)).to(torch.bfloat16)
+    # independent closed form in numpy float64 on the fp32 sum
+    s32 = (x.float() + r.float()).numpy().astype(np.float32)
+    s64 = s32.astype(np.float64)
+    y64 = s64 / np.sqrt((s64 ** 2).mean(-1, keepdims=True) + 1e-6)
+    ref = torch.from_numpy(y64.astype(np.float32)).to(torch.bfloat16) * w
+    got, res = orc.add_rmsnorm(x, r, w, 1e-6)
+    assert torch.equal(res, torch.from_numpy(s32).to(torch.bfloat16))
+    ulp = (got.view(torch.int16).int() - ref.view(torch.int16).int()).abs()
+    assert ulp.max() <= 1 and (ulp > 0).float().mean() < 2e-3
+    # statistics over the ROUNDED residual would be a different function
+    wrong = orc.rmsnorm(res, w, 1e-6)
+    assert (wrong != got).float().mean() > 0.01
+    # residual = 0 reduces it to the plain RMSNorm
+    z = torch.zeros_like(x)
+    got0, res0 = orc.add_rmsnorm(x, z, w, 1e-6)
+    assert torch.equal(got0, orc.rmsnorm(x, w, 1e-6)) and torch.equal(res0, x)
+
+
 def test_moe_only_layer_wiring():
     # decoder_layer.py:126-140 without attention: out = h + moe(norm(h))
     H, I, E, K, T = 128, 128, 4, 2, 6
