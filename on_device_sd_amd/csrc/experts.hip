@@ -397,6 +397,9 @@ struct ExpertsPlan {
     int NB;          // 16-row weight blocks per wavefront
     int WK_gu, WK_dn;  // wavefronts splitting K inside a workgroup (MB == 1 path)
     int KS;          // split of the down projection's reduction dimension across workgroups
+    int PS_gu, PS_dn;  // prefill tile kernel: workgroups sharing the row passes of one tile
+    int tile;        // MB == 8: the 256 x 256 tile kernel instead of the streaming kernel
+    int stream_nb4;  // MB == 8 streaming: 4 weight blocks per wavefront (comparison runs only)
     int y_f16;       // down-projection outputs kept as fp16 (prefill tile kernel) instead of fp32 partials
     size_t h_bytes, y_bytes;
 };
@@ -409,18 +412,28 @@ static ExpertsPlan experts_plan(const odsd_moe_shape *s) {
     const long P = (long)s->T * s->K;
     const long mean_rows = (P + s->E - 1) / s->E;
     // token blocks per pass follow the mean number of rows per expert; an expert with more
-    // rows than one pass holds takes further passes over its weights
+    // rows than one pass holds takes further passes over its weights.  Measured crossovers
+    // (uniform routing, Mixtral and Qwen3-235B expert shapes): 64-row passes win up to ~60 rows
+    // per expert, 128-row streaming passes up to ~130, the 256-row tile kernel beyond.
+    p.tile = 0;
     if (s->T <= 16) p.MB = 1;
     else if (s->T <= 32 || mean_rows <= 16) p.MB = 2;
-    else p.MB = (mean_rows * 3 / 2 <= 64) ? 4 : 8;
+    else if (mean_rows <= 52) p.MB = 4;
+    else { p.MB = 8; p.tile = mean_rows > 136; }
+    // tuning overrides for experiments: ODSD_GEMM_MB (1, 2, 4, 8), ODSD_GEMM_PREFILL (with 8 token
+    // blocks: 1 tile kernel, 2 streaming kernel, 0 streaming kernel with 4 weight blocks per wavefront)
     static const int env_mb = getenv("ODSD_GEMM_MB") ? atoi(getenv("ODSD_GEMM_MB")) : 0;
-    if (env_mb >= 1 && env_mb <= 4) p.MB = env_mb;
+    if (env_mb == 1 || env_mb == 2 || env_mb == 4 || env_mb == 8) { p.MB = env_mb; p.tile = env_mb == 8 && mean_rows > 136; }
+    static const int env_pf = getenv("ODSD_GEMM_PREFILL") ? atoi(getenv("ODSD_GEMM_PREFILL")) : -1;
+    p.stream_nb4 = 0;
+    if (p.MB == 8 && env_pf >= 0) { p.tile = env_pf == 1; p.stream_nb4 = env_pf == 0; }
     const long active = s->E < P ? s->E : P;       // upper bound of experts with rows
     const long slots = 512;                        // 256 CUs x 2 workgroups
     const int G_gu = s->H / ODSD_GROUP, G_dn = s->I / ODSD_GROUP;
     p.NB = 4;
     p.WK_gu = p.WK_dn = 1;
     p.KS = 1;
+    p.PS_gu = p.PS_dn = 1;
     if (p.MB == 1) {
         // many small work items: 4 wavefronts split K when each still gets >= 2 groups
         p.WK_gu = G_gu >= 8 ? 4 : (G_gu >= 4 ? 2 : 1);
@@ -430,17 +443,30 @@ static ExpertsPlan experts_plan(const odsd_moe_shape *s) {
         p.KS = KS;
         const int gper = (G_dn + KS - 1) / KS;
         p.WK_dn = gper >= 8 ? 4 : (gper >= 4 ? 2 : 1);
-    } else if (p.MB >= 8) {
-        p.KS = 1;      // the prefill tile kernel reduces over the whole of I
+    } else if (p.tile) {
+        // 256 x 256 tiles: with few experts the tiles alone do not fill 256 CUs.  First hand the
+        // row passes of one tile (it re-reads its weights per pass anyway) to several workgroups,
+        // then split the down projection's reduction.
+        const long mean_passes = (mean_rows + 255) / 256;
+        const long tiles_gu = active * ((2 * s->I / 16 + 15) / 16), tiles_dn = active * ((s->H / 16 + 15) / 16);
+        while (tiles_gu * p.PS_gu < slots && p.PS_gu * 2 <= mean_passes) p.PS_gu *= 2;
+        while (tiles_dn * p.PS_dn < slots && p.PS_dn * 2 <= mean_passes) p.PS_dn *= 2;
+        int KS = 1;
+        while (tiles_dn * p.PS_dn * KS < slots && KS * 2 <= G_dn / 4 && KS < 16) KS *= 2;
+        p.KS = KS;
     } else {
         if (p.MB <= 4) {
             const long wg_gu = active * ((2 * s->I / 16 + 15) / 16);
             if (wg_gu < 4 * slots) p.NB = 2;
             if (env_nb == 2 || env_nb == 4) p.NB = env_nb;
+        } else {
+            p.NB = p.stream_nb4 ? 4 : 2;
         }
         const int nchunks_dn = (s->H / 16 + 4 * p.NB - 1) / (4 * p.NB);
+        // up to 4 workgroups per CU with at most 4 token blocks, 2 with 8
+        const long want = p.MB <= 4 ? 2 * slots : slots;
         int KS = 1;
-        while (KS * 2 <= G_dn / 2 && active * nchunks_dn * KS < 2 * slots && KS < 16) KS *= 2;
+        while (KS * 2 <= G_dn / 2 && active * nchunks_dn * KS < want && KS < 16) KS *= 2;
         p.KS = KS;
     }
     static const int env_ks = getenv("ODSD_GEMM_KS") ? atoi(getenv("ODSD_GEMM_KS")) : 0;
@@ -449,8 +475,7 @@ static ExpertsPlan experts_plan(const odsd_moe_shape *s) {
     while (p.KS > 1 && ((G_dn + p.KS - 1) / p.KS) * (p.KS - 1) >= G_dn) p.KS--;
     // At prefill shapes the fp32 partials would be 0.5 GB written and read back per layer; fp16
     // still carries 3 more bits than the bf16 the reference keeps its expert outputs in.
-    static const int env_pf = getenv("ODSD_GEMM_PREFILL") ? atoi(getenv("ODSD_GEMM_PREFILL")) : 1;
-    p.y_f16 = p.MB >= 8 && env_pf == 1 && p.KS == 1;
+    p.y_f16 = p.tile && p.KS == 1;
     p.h_bytes = odsd_round_up((size_t)(P > 0 ? P : 1) * s->I * sizeof(half_t), 256);
     p.y_bytes = odsd_round_up((size_t)p.KS * (size_t)(P > 0 ? P : 1) * s->H * sizeof(float), 256);
     return p;
@@ -495,12 +520,12 @@ static void launch_gemm_plan(const ExpertsPlan &pl, GemmParams &gp, hipStream_t 
     } else if (pl.MB == 4) {
         if (pl.NB == 2) launch_gemm<2, 4, MODE, 2, 2, 1, false, 4>(gp, st);
         else launch_gemm<4, 4, MODE, 2, 2, 1, false, 2>(gp, st);
-    } else {
-        // ODSD_GEMM_PREFILL=0 keeps the streaming kernel (for comparison runs)
-        static const int v = getenv("ODSD_GEMM_PREFILL") ? atoi(getenv("ODSD_GEMM_PREFILL")) : 1;
+    } else if (pl.tile) {
         gp.y_f16 = pl.y_f16;
-        if (v == 1) odsd_launch_gemm_prefill<MODE>(gp, st);
-        else launch_gemm<4, 8, MODE, 2, 4, 1, false, 1>(gp, st);
+        odsd_launch_gemm_prefill<MODE>(gp, st);
+    } else {
+        if (pl.stream_nb4) launch_gemm<4, 8, MODE, 2, 4, 1, false, 1>(gp, st);
+        else launch_gemm<2, 8, MODE, 2, 2, 1, false, 2>(gp, st);
     }
 }
 
@@ -523,7 +548,7 @@ extern "C" int odsd_w4_gate_up_silu(const odsd_moe_shape *s, const void *x_f16, 
     gu.table = table; gu.src = (const half_t *)x_f16; gu.rowmap = slot_token;
     gu.counts = counts; gu.offsets = offsets; gu.h16 = (half_t *)h_f16; gu.y = nullptr;
     gu.src_ld = s->H; gu.G = s->H / ODSD_GROUP; gu.NBLK = 2 * s->I / 16;
-    gu.KS = 1; gu.gper = gu.G; gu.ldo = s->I; gu.P = s->T * s->K; gu.E = s->E;
+    gu.KS = 1; gu.gper = gu.G; gu.PS = pl.PS_gu; gu.ldo = s->I; gu.P = s->T * s->K; gu.E = s->E;
     launch_gemm_plan<0>(pl, gu, (hipStream_t)stream);
     ODSD_CHECK_LAUNCH();
     return ODSD_OK;
@@ -547,7 +572,7 @@ extern "C" int odsd_w4_down(const odsd_moe_shape *s, const void *h_f16, const ui
     dn.table = table; dn.src = (const half_t *)h_f16; dn.rowmap = nullptr;
     dn.counts = counts; dn.offsets = offsets; dn.h16 = nullptr; dn.y = (float *)y;
     dn.src_ld = s->I; dn.G = s->I / ODSD_GROUP; dn.NBLK = s->H / 16;
-    dn.KS = pl.KS; dn.gper = (dn.G + pl.KS - 1) / pl.KS; dn.ldo = s->H; dn.P = s->T * s->K; dn.E = s->E;
+    dn.KS = pl.KS; dn.gper = (dn.G + pl.KS - 1) / pl.KS; dn.PS = pl.PS_dn; dn.ldo = s->H; dn.P = s->T * s->K; dn.E = s->E;
     launch_gemm_plan<1>(pl, dn, (hipStream_t)stream);
     ODSD_CHECK_LAUNCH();
     return ODSD_OK;

@@ -41,8 +41,11 @@ __global__ __launch_bounds__(512, 2) void w4_gemm_prefill_kernel(const GemmParam
     const int b = blockIdx.x;
     const int L = (b & 7) * p.wg_per_xcd + (b >> 3);
     if (L >= p.n_wg) return;
+    // row chunks innermost: neighbours share the token rows of one (expert, pass, K slice)
     const int chunk = L % p.nchunks;
-    const int e = L / p.nchunks;
+    const int ks = (L / p.nchunks) % p.KS;
+    const int ps = (L / (p.nchunks * p.KS)) % p.PS;
+    const int e = L / (p.nchunks * p.KS * p.PS);
 
     const int M_e = p.counts[e];
     if (M_e == 0) return;
@@ -60,6 +63,7 @@ __global__ __launch_bounds__(512, 2) void w4_gemm_prefill_kernel(const GemmParam
     const int wn = wave & 3, wm = wave >> 2;
     const int G = p.G;
     const int NST = 2 * G;                     // stages of 64 columns
+    const int g_begin = ks * p.gper, g_end = min(G, g_begin + p.gper);   // this K slice (never empty)
 
     // expansion duty: tiles 2*wave and 2*wave+1 of this row chunk (clamped, never out of range)
     uint32_t wq_off[2], sz_off[2];
@@ -76,7 +80,7 @@ __global__ __launch_bounds__(512, 2) void w4_gemm_prefill_kernel(const GemmParam
 #pragma unroll
     for (int i = 0; i < 4; ++i) blk_ok[i] = cblk0 + i < p.NBLK;
 
-    for (int m0 = 0; m0 < M_e; m0 += BM) {
+    for (int m0 = ps * BM; m0 < M_e; m0 += p.PS * BM) {
         const int mcnt = min(M_e - m0, BM);
         const int mrows_w = max(0, min(mcnt - wm * 16 * MBW, 16 * MBW));   // rows of this M half
         const int nmb = (mrows_w + 15) >> 4;
@@ -220,9 +224,9 @@ __global__ __launch_bounds__(512, 2) void w4_gemm_prefill_kernel(const GemmParam
 
         // prologue: stage 0 in place
         __builtin_amdgcn_s_barrier();          // the previous pass is done with both LDS areas
-        dma_x(xs0, 0);
-        load_w(0, 0);
-        load_w(1, 1);
+        dma_x(xs0, 2 * g_begin);
+        load_w(0, g_begin);
+        load_w(1, g_begin + 1);
         __builtin_amdgcn_sched_barrier(0);
         expand(0, 0, ws0);
         __builtin_amdgcn_sched_barrier(0);
@@ -230,7 +234,7 @@ __global__ __launch_bounds__(512, 2) void w4_gemm_prefill_kernel(const GemmParam
         __builtin_amdgcn_s_barrier();
 
         // two groups (four stages) per trip: ring slots and buffers are compile-time constants
-        for (int g = 0; g < G; g += 2) {
+        for (int g = g_begin; g < g_end; g += 2) {
             // stage 4k   : group g, first half.   produce (g, second half) -> x buf 1, w buf 1
             dma_x(xs1, 2 * g + 1);
             __builtin_amdgcn_sched_barrier(0);
@@ -247,7 +251,7 @@ __global__ __launch_bounds__(512, 2) void w4_gemm_prefill_kernel(const GemmParam
             __builtin_amdgcn_sched_barrier(0);
             ODSD_WAIT_VMCNT_LGKM0(0);
             __builtin_amdgcn_s_barrier();
-            if (g + 1 >= G) break;
+            if (g + 1 >= g_end) break;
             // stage 4k+2 : group g+1, first half.  produce (g+1, second half) -> buffers 1
             dma_x(xs1, 2 * g + 3);
             __builtin_amdgcn_sched_barrier(0);
@@ -296,7 +300,7 @@ __global__ __launch_bounds__(512, 2) void w4_gemm_prefill_kernel(const GemmParam
                                 *(half4_t *)((half_t *)p.y + slot * p.ldo + n) =
                                     half4_t{f32_to_f16_sat(v.x), f32_to_f16_sat(v.y), f32_to_f16_sat(v.z), f32_to_f16_sat(v.w)};
                             } else {
-                                *(float4_t *)(p.y + slot * p.ldo + n) = acc[i][m];
+                                *(float4_t *)(p.y + ((size_t)ks * p.P + slot) * p.ldo + n) = acc[i][m];
                             }
                         }
                     }
@@ -309,7 +313,8 @@ __global__ __launch_bounds__(512, 2) void w4_gemm_prefill_kernel(const GemmParam
 template <int MODE>
 void odsd_launch_gemm_prefill(GemmParams &gp, hipStream_t st) {
     gp.nchunks = (gp.NBLK + 15) / 16;
-    gp.n_wg = gp.E * gp.nchunks;
+    if (gp.PS < 1) gp.PS = 1;
+    gp.n_wg = gp.E * gp.nchunks * gp.KS * gp.PS;
     gp.wg_per_xcd = (gp.n_wg + 7) / 8;
     w4_gemm_prefill_kernel<MODE, 8><<<gp.wg_per_xcd * 8, 512, 0, st>>>(gp);
 }

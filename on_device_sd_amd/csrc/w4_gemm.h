@@ -23,10 +23,11 @@ struct GemmParams {
     int nchunks;             // workgroup tiles along the rows
     int KS;                  // splits of the reduction dimension
     int gper;                // groups per split
+    int PS;                  // prefill tile kernel: workgroups sharing the row passes of one tile
     int ldo;                 // I (MODE 0) or H (MODE 1)
     int P;
     int E;
-    int n_wg;                // E * nchunks * KS
+    int n_wg;                // E * nchunks * KS (* PS)
     int wg_per_xcd;          // ceil(n_wg / 8)
 };
 

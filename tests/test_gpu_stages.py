@@ -158,10 +158,13 @@ EXPERT_CASES = [
     (70, 384, 4, 2, 640, torch.bfloat16),     # >16 rows per expert, ragged row blocks (I/16 = 40)
     (200, 256, 2, 2, 256, torch.bfloat16),    # 200 rows per expert: several passes
     (64, 2048, 128, 8, 768, torch.bfloat16),  # config 3 shape (uniform routing)
-    # prefill tile kernel (mean rows per expert > 42) at awkward sizes:
+    (390, 384, 3, 1, 640, torch.bfloat16),    # 130 rows per expert on average: 128-row streaming passes, some experts two
+    # prefill tile kernel (mean rows per expert > 136) at awkward sizes:
     (700, 384, 3, 2, 384, torch.bfloat16),    # odd group count, 1.5 row chunks in down, 2 passes per expert
     (300, 640, 2, 1, 128, torch.float32),     # top-1, a single group in down, 2.5 row chunks, fp32 activations
-    (100, 256, 2, 2, 128, torch.bfloat16),    # 100 rows per expert: one partial pass
+    (100, 256, 2, 2, 128, torch.bfloat16),    # 100 rows per expert: one partial 128-row streaming pass
+    (600, 256, 2, 2, 1024, torch.bfloat16),   # few tiles: passes shared by workgroups, down reduction split in 2
+    (260, 256, 1, 1, 1280, torch.bfloat16),   # one expert, 10 groups in down: two slices of 5 (odd start, odd length)
 ]
 
 
