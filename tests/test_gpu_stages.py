@@ -158,6 +158,8 @@ EXPERT_CASES = [
     (70, 384, 4, 2, 640, torch.bfloat16),     # >16 rows per expert, ragged row blocks (I/16 = 40)
     (200, 256, 2, 2, 256, torch.bfloat16),    # 200 rows per expert: several passes
     (64, 2048, 128, 8, 768, torch.bfloat16),  # config 3 shape (uniform routing)
+    (100, 256, 4, 2, 384, torch.bfloat16),    # 64-row passes (some experts two), 3 groups in down
+    (24, 384, 4, 2, 256, torch.float32),      # 32-row passes, 2 groups in down, 3 row chunks
     (390, 384, 3, 1, 640, torch.bfloat16),    # 130 rows per expert on average: 128-row streaming passes, some experts two
     # prefill tile kernel (mean rows per expert > 136) at awkward sizes:
     (700, 384, 3, 2, 384, torch.bfloat16),    # odd group count, 1.5 row chunks in down, 2 passes per expert
