@@ -47,12 +47,7 @@ def _build_layer(wl, dev, layer=0):
 
 
 def _clone_bank(bank):
-    import on_device_sd_amd as odsd
-    b = odsd.W4ExpertBank.__new__(odsd.W4ExpertBank)
-    b.__dict__.update(bank.__dict__)
-    b.gu_q, b.gu_sz, b.dn_q, b.dn_sz = (t.clone() for t in (bank.gu_q, bank.gu_sz, bank.dn_q, bank.dn_sz))
-    b._table = None
-    return b
+    return bank.clone()
 
 
 def _event_ms(fn, n):
@@ -108,6 +103,31 @@ def bench_layer(wl, dev, steps, warmup, with_cpu):
     k_rt = _event_ms(lambda i: ops.router_topk(x, gate, wl.K, wl.renorm, want_f16=True), n)
     k_dp = _event_ms(lambda i: ops.dispatch(idx, wl.E), n)
 
+    # the two-call path of the reference engine loops: route_experts, the host reads the
+    # activated set, forward_moe (reported beside the whole-block call, never as `value`)
+    import on_device_sd_amd as odsd
+    cfg = odsd.MoEConfig(hidden_size=wl.H, num_hidden_layers=n_rep, num_experts=wl.E,
+                         num_experts_per_token=wl.K, moe_intermediate_size=wl.I, norm_topk_prob=wl.renorm,
+                         torch_dtype="float32" if wl.act_dtype == torch.float32 else "bfloat16")
+    runner = odsd.W4MoERunner(cfg, [gate] * n_rep, banks)
+    placements = [odsd.ExpertPlacement(gpu_expert_params=b.all_expert_params(), cpu_expert_params={})
+                  for b in banks]
+
+    def engine_step(i):
+        l = i % n_rep
+        placements[l].routing_result = runner.route_experts(l, x)
+        runner.forward_moe(l, odsd.AttentionOutput(hidden_states=x, post_attn_normed=x, residual=x),
+                           placements[l])
+
+    for i in range(max(3, warmup)):
+        engine_step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(n):
+        engine_step(i)
+    torch.cuda.synchronize()
+    engine_ms = (time.perf_counter() - t0) * 1e3 / n
+
     gu_bytes = active * (wl.expert_w4_bytes * 2 // 3)
     gu_flops = 4 * wl.pairs * wl.H * wl.I
     if wl.regime == "prefill":
@@ -125,7 +145,8 @@ def bench_layer(wl, dev, steps, warmup, with_cpu):
     layer_bytes_alg = wl.algorithmic_bytes(active)
     res = {
         "workload": wl.name, "T": wl.T, "H": wl.H, "E": wl.E, "K": wl.K, "I": wl.I,
-        "tokens_per_s": wl.T / (ms * 1e-3), "ms_per_step": ms, "active_experts": active,
+        "tokens_per_s": wl.T / (ms * 1e-3), "ms_per_step": ms, "engine_path_ms": engine_ms,
+        "active_experts": active,
         "max_rows_per_expert": int(counts.max()), "weight_replicas": n_rep,
         "layer_hbm_frac": layer_bytes_alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "layer_mfma_frac": wl.algorithmic_flops() / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS,

@@ -8,19 +8,17 @@ code written against the reference works unchanged on top of this runner.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Dict, Optional, Set
+from typing import Any, Dict, NamedTuple, Optional, Set, Tuple
 
 import torch
 
 
-@dataclass
-class ExpertID:
-    """Unique identifier of an expert (types.py:19-29)."""
+class ExpertID(NamedTuple):
+    """Unique identifier of an expert (types.py:19-29): same fields, construction, equality and
+    string form as the reference's dataclass.  A named tuple hashes and compares in C, which
+    matters where a set of up to E of them is built per layer and step."""
     layer_idx: int
     expert_idx: int
-
-    def __hash__(self):
-        return hash((self.layer_idx, self.expert_idx))
 
     def __str__(self):
         return f"L{self.layer_idx}_E{self.expert_idx}"
@@ -33,13 +31,17 @@ class RoutingResult:
     topk_indices [T, K] int64 in descending-score order, topk_scores [T, K] float32.
     ``dispatch`` is an optional cache of the device-side dispatch arrays that
     route_experts already produced; forward_moe recomputes them when it is absent
-    (for example on a hand-built RoutingResult).
+    (for example on a hand-built RoutingResult).  ``x_f16`` is the fp16 copy of the routed
+    hidden states that the router kernel writes anyway, tagged with the identity of the tensor
+    it was made from; forward_moe uses it when it is handed that same, unmodified tensor.
     """
     layer_idx: int
     topk_indices: torch.Tensor
     topk_scores: torch.Tensor
     activated_expert_ids: Set[ExpertID]
     dispatch: Optional[Any] = field(default=None, repr=False, compare=False)
+    x_f16: Optional[torch.Tensor] = field(default=None, repr=False, compare=False)
+    x_tag: Optional[Tuple] = field(default=None, repr=False, compare=False)
 
     @property
     def top_k(self) -> int:

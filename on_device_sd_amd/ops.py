@@ -164,9 +164,10 @@ class Dispatch:
     perm: torch.Tensor        # int32 [P]  pair -> slot
     inv: torch.Tensor         # int32 [P]  slot -> pair
     slot_token: torch.Tensor  # int32 [P]  slot -> token
+    idx32: Optional[torch.Tensor] = None   # the int32 [T, K] indices the arrays were built from
 
 
-def dispatch(idx: torch.Tensor, num_experts: int) -> Dispatch:
+def dispatch(idx: torch.Tensor, num_experts: int, idx32_keep: bool = False) -> Dispatch:
     _require_cuda(idx)
     lib = _lib.load()
     if idx.dtype != torch.int32:
@@ -175,11 +176,13 @@ def dispatch(idx: torch.Tensor, num_experts: int) -> Dispatch:
     T, K = idx.shape
     dev = idx.device
     shape = MoeShape(T, 128, num_experts, K, 128, 0, _lib.DT_F32, 0)
-    d = Dispatch(torch.empty(num_experts, dtype=torch.int32, device=dev),
-                 torch.empty(num_experts + 1, dtype=torch.int32, device=dev),
-                 torch.empty(T * K, dtype=torch.int32, device=dev),
-                 torch.empty(T * K, dtype=torch.int32, device=dev),
-                 torch.empty(T * K, dtype=torch.int32, device=dev))
+    # one allocation, five views (each 16-byte aligned)
+    P = T * K
+    e_pad, e1_pad, p_pad = (num_experts + 3) & ~3, (num_experts + 4) & ~3, (P + 3) & ~3
+    buf = torch.empty(e_pad + e1_pad + 3 * p_pad, dtype=torch.int32, device=dev)
+    o1, o2, o3, o4 = e_pad, e_pad + e1_pad, e_pad + e1_pad + p_pad, e_pad + e1_pad + 2 * p_pad
+    d = Dispatch(buf[:num_experts], buf[o1:o1 + num_experts + 1], buf[o2:o2 + P], buf[o3:o3 + P],
+                 buf[o4:o4 + P], idx if idx32_keep else None)
     if T == 0:
         d.counts.zero_()
         d.offsets.zero_()

@@ -45,7 +45,14 @@ class W4MoERunner:
         self.banks = banks
         self.norm_weights = None if norm_weights is None else [
             n.to(device=self.device, dtype=self.dtype).contiguous() for n in norm_weights]
-        self._table_cache: Dict[tuple, torch.Tensor] = {}
+        self._table_cache: Dict[tuple, tuple] = {}
+        # host side of the hop between routing and execution: a pinned landing buffer for the E
+        # counts, an event to wait for just that copy, and the ExpertID objects made once
+        E = config.num_experts
+        self._counts_host = torch.empty(E, dtype=torch.int32, pin_memory=True)
+        self._counts_np = self._counts_host.numpy()
+        self._counts_event = torch.cuda.Event()
+        self._expert_ids = [[ExpertID(l, e) for e in range(E)] for l in range(len(banks))]
 
     # -- ModelRunner interface -----------------------------------------------------------------
     def get_config(self) -> MoEConfig:
@@ -57,16 +64,22 @@ class W4MoERunner:
     def route_experts(self, layer_idx: int, hidden_states: torch.Tensor) -> RoutingResult:
         cfg = self.config
         flat = hidden_states.reshape(-1, hidden_states.shape[-1])
-        idx32, w, idx64, _ = ops.router_topk(flat, self.gate_weights[layer_idx],
-                                             cfg.num_experts_per_token, cfg.norm_topk_prob,
-                                             want_int64=True)
-        disp = ops.dispatch(idx32, cfg.num_experts)
+        idx32, w, idx64, x16 = ops.router_topk(flat, self.gate_weights[layer_idx],
+                                               cfg.num_experts_per_token, cfg.norm_topk_prob,
+                                               want_f16=True, want_int64=True)
+        disp = ops.dispatch(idx32, cfg.num_experts, idx32_keep=True)
         # the engine reads the activated set on the host between routing and execution
-        # (qwen3_runner.py:110-112): one small device-to-host copy of the E counts
-        counts = disp.counts.cpu().tolist()
-        activated = {ExpertID(layer_idx, e) for e, c in enumerate(counts) if c > 0}
+        # (qwen3_runner.py:110-112): one asynchronous copy of the E counts into pinned memory,
+        # and a wait for that copy alone
+        self._counts_host.copy_(disp.counts, non_blocking=True)
+        self._counts_event.record()
+        self._counts_event.synchronize()
+        ids = self._expert_ids[layer_idx] if layer_idx < len(self._expert_ids) else \
+            [ExpertID(layer_idx, e) for e in range(cfg.num_experts)]
+        activated = set(map(ids.__getitem__, self._counts_np.nonzero()[0].tolist()))
         return RoutingResult(layer_idx=layer_idx, topk_indices=idx64, topk_scores=w,
-                             activated_expert_ids=activated, dispatch=disp)
+                             activated_expert_ids=activated, dispatch=disp, x_f16=x16,
+                             x_tag=_tensor_tag(flat))
 
     def forward_moe(self, layer_idx: int, attn_output: AttentionOutput,
                     expert_placement: ExpertPlacement) -> torch.Tensor:
@@ -97,22 +110,28 @@ class W4MoERunner:
 
     # -- internals -----------------------------------------------------------------------------
     def _placement_table(self, placement: ExpertPlacement) -> torch.Tensor:
+        """Device pointer table of a placement.  Placements repeat from step to step, so tables
+        are cached; the key is built from the identities of the parameter objects (a bank hands
+        out one object per expert), and the cache entry keeps those objects alive so that an
+        identity cannot be reused while the entry exists."""
+        gpu, cpu, sub = placement.gpu_expert_params, placement.cpu_expert_params, placement.substitution_map
+        key = (tuple(gpu), tuple(map(id, gpu.values())), tuple(cpu), tuple(map(id, cpu.values())),
+               tuple(sub.items()) if sub else ())
+        hit = self._table_cache.get(key)
+        if hit is not None:
+            return hit[0]
         params: Dict[int, W4ExpertParams] = {}
-        for src in (placement.gpu_expert_params, placement.cpu_expert_params):
+        for src in (gpu, cpu):
             for e, p in src.items():
                 if not isinstance(p, W4ExpertParams):
                     raise TypeError(
                         f"expert {e}: parameters are not W4 bundles resident in HBM; this runner "
                         "executes every expert on the GPU and has no CPU expert path")
                 params[e] = p
-        key = (tuple(sorted((e, p.ptrs) for e, p in params.items())),
-               tuple(sorted(placement.substitution_map.items())))
-        tab = self._table_cache.get(key)
-        if tab is None:
-            if len(self._table_cache) > 64:
-                self._table_cache.clear()
-            tab = build_table(self.config.num_experts, params, placement.substitution_map, self.device)
-            self._table_cache[key] = tab
+        if len(self._table_cache) > 64:
+            self._table_cache.clear()
+        tab = build_table(self.config.num_experts, params, sub, self.device)
+        self._table_cache[key] = (tab, list(gpu.values()), list(cpu.values()))
         return tab
 
     def _execute_moe_with_placement(self, hidden_states: torch.Tensor, placement: ExpertPlacement,
@@ -129,13 +148,24 @@ class W4MoERunner:
         if disp is None:
             idx = idx.to(device=flat.device, dtype=torch.int32)
             disp = ops.dispatch(idx, self.config.num_experts)
+        elif disp.idx32 is not None:
+            idx = disp.idx32          # the router's own int32 indices: no conversion kernel
         scores = routing.topk_scores.reshape(flat.shape[0], -1).to(device=flat.device,
                                                                   dtype=torch.float32)
         table = self._placement_table(placement)
-        _, out = ops.experts_w4(ops.to_f16(flat), table, idx, scores, disp,
+        # the fp16 copy the router wrote, if these are the very hidden states it routed
+        x16 = routing.x_f16 if routing.x_f16 is not None and routing.x_tag == _tensor_tag(flat) \
+            else ops.to_f16(flat)
+        _, out = ops.experts_w4(x16, table, idx, scores, disp,
                                 self.config.moe_intermediate_size, flat.dtype, residual=res,
                                 want_f32=False, want_act=True)
         return out.view(shape)
+
+
+def _tensor_tag(t: torch.Tensor) -> tuple:
+    """Identity of a tensor's contents as far as the host can tell: storage address, shape,
+    dtype and the in-place modification counter."""
+    return (t.data_ptr(), tuple(t.shape), t.dtype, t._version)
 
 
 # -- stateless forms ---------------------------------------------------------------------------

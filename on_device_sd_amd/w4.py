@@ -46,10 +46,7 @@ class W4ExpertParams(dict):
                          down_proj=W4Proj(bank, expert, "down_proj", (H, I)))
         self.bank = bank
         self.expert = expert
-
-    @property
-    def ptrs(self) -> Tuple[int, int, int, int]:
-        return self.bank.expert_ptrs(self.expert)
+        self.ptrs: Tuple[int, int, int, int] = bank.expert_ptrs(expert)
 
 
 class W4ExpertBank:
@@ -65,7 +62,26 @@ class W4ExpertBank:
         self.gu_q, self.gu_sz = mk(self.gu_q_bytes), mk(self.gu_sz_bytes)
         self.dn_q, self.dn_sz = mk(self.dn_q_bytes), mk(self.dn_sz_bytes)
         self.loaded = [False] * E
+        self._bind_storage()
+
+    def _bind_storage(self) -> None:
+        """The storage never moves: addresses and parameter objects are made once per bank."""
         self._table: Optional[torch.Tensor] = None
+        self._ptrs = [(self.gu_q[e].data_ptr(), self.gu_sz[e].data_ptr(),
+                       self.dn_q[e].data_ptr(), self.dn_sz[e].data_ptr())
+                      for e in range(self.num_experts)]
+        self._params: Dict[int, W4ExpertParams] = {}
+
+    def clone(self) -> "W4ExpertBank":
+        """A second copy of the packed weights in HBM (same contents, its own storage)."""
+        b = W4ExpertBank.__new__(W4ExpertBank)
+        b.num_experts, b.hidden, b.inter, b.device = self.num_experts, self.hidden, self.inter, self.device
+        b.gu_q_bytes, b.gu_sz_bytes = self.gu_q_bytes, self.gu_sz_bytes
+        b.dn_q_bytes, b.dn_sz_bytes = self.dn_q_bytes, self.dn_sz_bytes
+        b.gu_q, b.gu_sz, b.dn_q, b.dn_sz = (t.clone() for t in (self.gu_q, self.gu_sz, self.dn_q, self.dn_sz))
+        b.loaded = list(self.loaded)
+        b._bind_storage()
+        return b
 
     # -- sizes -------------------------------------------------------------------------------
     @property
@@ -118,13 +134,17 @@ class W4ExpertBank:
 
     # -- views -------------------------------------------------------------------------------
     def expert_ptrs(self, e: int) -> Tuple[int, int, int, int]:
-        return (self.gu_q[e].data_ptr(), self.gu_sz[e].data_ptr(),
-                self.dn_q[e].data_ptr(), self.dn_sz[e].data_ptr())
+        return self._ptrs[e]
 
     def expert_params(self, e: int) -> W4ExpertParams:
+        """The parameter dict of expert e: one object per expert for the life of the bank, so
+        that a placement can be recognised by the identity of its values."""
         if not self.loaded[e]:
             raise KeyError(f"expert {e} has not been loaded")
-        return W4ExpertParams(self, e)
+        p = self._params.get(e)
+        if p is None:
+            p = self._params[e] = W4ExpertParams(self, e)
+        return p
 
     def all_expert_params(self) -> Dict[int, W4ExpertParams]:
         return {e: self.expert_params(e) for e in range(self.num_experts) if self.loaded[e]}

@@ -161,6 +161,51 @@ def test_route_then_forward_equals_whole_block_and_oracle(runner, dev):
                                         E, K, I, return_f32=True).reshape(-1, H), ref)
 
 
+def test_router_fp16_copy_is_reused_only_for_the_routed_tensor(runner, dev):
+    import on_device_sd_amd as odsd
+    hidden = _hidden(dev, 7, H, seed=5)
+    res = runner.route_experts(0, hidden)
+    assert res.x_f16 is not None and torch.equal(res.x_f16, hidden.to(torch.float16))
+    params = runner.banks[0].all_expert_params()
+    idx, sc = res.topk_indices.cpu().numpy(), res.topk_scores.cpu().numpy()
+
+    def run(h):
+        placement = odsd.ExpertPlacement(gpu_expert_params=params, cpu_expert_params={}, routing_result=res)
+        return runner.forward_moe(0, _attn(h), placement)
+
+    out_same = run(hidden)
+    check_output(out_same, orc.forward_moe(hidden.cpu(), hidden.cpu(), idx, sc, runner.oracle_experts[0]))
+    # other hidden states with the same routing: the cached copy must not be used
+    other = _hidden(dev, 7, H, seed=6)
+    check_output(run(other), orc.forward_moe(other.cpu(), other.cpu(), idx, sc, runner.oracle_experts[0]))
+    # the routed tensor modified in place after routing: its version counter has moved on
+    hidden.mul_(0.5)
+    check_output(run(hidden), orc.forward_moe(hidden.cpu(), hidden.cpu(), idx, sc, runner.oracle_experts[0]))
+
+
+def test_placement_tables_are_cached_by_parameter_identity(runner, dev):
+    import on_device_sd_amd as odsd
+    bank = runner.banks[0]
+    assert bank.expert_params(1) is bank.expert_params(1)
+    p1 = odsd.ExpertPlacement(gpu_expert_params=bank.all_expert_params(), cpu_expert_params={})
+    p2 = odsd.ExpertPlacement(gpu_expert_params=bank.all_expert_params(), cpu_expert_params={})
+    t1, t2 = runner._placement_table(p1), runner._placement_table(p2)
+    assert t1 is t2 and torch.equal(t1.cpu(), bank.table().cpu())
+    # a different set of experts, a substitution, or another bank's parameters give other tables
+    p3 = odsd.ExpertPlacement(gpu_expert_params={0: bank.expert_params(0)}, cpu_expert_params={})
+    p4 = odsd.ExpertPlacement(gpu_expert_params={0: bank.expert_params(0)}, cpu_expert_params={},
+                              substitution_map={1: 0})
+    p5 = odsd.ExpertPlacement(gpu_expert_params={0: runner.banks[1].expert_params(0)}, cpu_expert_params={})
+    t3, t4, t5 = (runner._placement_table(p).cpu() for p in (p3, p4, p5))
+    assert t3[0].tolist() == list(bank.expert_ptrs(0)) and not t3[1:].any()
+    assert t4[1].tolist() == list(bank.expert_ptrs(0)) and not t4[2:].any()
+    assert t5[0].tolist() == list(runner.banks[1].expert_ptrs(0))
+    # a cloned bank has its own storage and its own addresses
+    clone = bank.clone()
+    assert clone.expert_ptrs(0) != bank.expert_ptrs(0)
+    assert torch.equal(clone.gu_q, bank.gu_q) and torch.equal(clone.table()[:, 0].cpu() != 0, bank.table()[:, 0].cpu() != 0)
+
+
 def test_forward_layer_metadata_and_wiring(runner, dev):
     hidden = _hidden(dev, 6, H, seed=4)
     lo = runner.forward_layer(0, hidden)
