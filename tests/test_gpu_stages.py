@@ -161,6 +161,13 @@ EXPERT_CASES = [
     (100, 256, 4, 2, 384, torch.bfloat16),    # 64-row passes (some experts two), 3 groups in down
     (24, 384, 4, 2, 256, torch.float32),      # 32-row passes, 2 groups in down, 3 row chunks
     (390, 384, 3, 1, 640, torch.bfloat16),    # 130 rows per expert on average: 128-row streaming passes, some experts two
+    # direct path (T <= 16): K split over 4 and over 2 wavefronts, and a down reduction split over workgroups
+    (8, 1024, 4, 2, 256, torch.bfloat16),
+    (5, 512, 4, 2, 1024, torch.float32),
+    (4, 256, 2, 1, 2048, torch.bfloat16),
+    # many experts with long rows: 4 weight blocks per wavefront, 32-row and 64-row passes
+    (40, 128, 128, 4, 2048, torch.bfloat16),
+    (300, 128, 128, 8, 2048, torch.bfloat16),
     # prefill tile kernel (mean rows per expert > 136) at awkward sizes:
     (700, 384, 3, 2, 384, torch.bfloat16),    # odd group count, 1.5 row chunks in down, 2 passes per expert
     (300, 640, 2, 1, 128, torch.float32),     # top-1, a single group in down, 2.5 row chunks, fp32 activations
