@@ -19,6 +19,7 @@
  * Reference interfaces each entry point stands in for (paths relative to the
  * potatoZhx/on_device_sd tree):
  *   odsd_router_topk   Qwen3MoEGate.forward                    demo/src/layers/moe_layer.py:25-60
+ *   odsd_router_topk_logits  + GPUOperators.router            demo/src/operators/gpu_operators.py:48-69
  *                      Qwen3ModelRunner.route_experts          demo/src/model/qwen3_runner.py:86-119
  *                      GPUOperators.router                     demo/src/operators/gpu_operators.py:48-69
  *   odsd_dispatch      mask / torch.where per expert           demo/src/model/qwen3_runner.py:303-314
@@ -119,6 +120,13 @@ size_t odsd_router_workspace_bytes(const odsd_moe_shape *s);
 int odsd_router_topk(const odsd_moe_shape *s, const void *x, const void *gate_w,
                      int32_t *out_idx, float *out_w, int64_t *out_idx64, void *x_f16,
                      void *workspace, size_t workspace_bytes, void *stream);
+/* The same, and the summed fp64 logits out_logits [T,E] (row-major) besides: the
+ * `scores = F.linear(flat_hidden, router_weight)` that GPUOperators.router returns
+ * (demo/src/operators/gpu_operators.py:48-69) and Qwen3MoEGate.forward computes first
+ * (demo/src/layers/moe_layer.py:44). */
+int odsd_router_topk_logits(const odsd_moe_shape *s, const void *x, const void *gate_w,
+                            int32_t *out_idx, float *out_w, int64_t *out_idx64, void *x_f16,
+                            double *out_logits, void *workspace, size_t workspace_bytes, void *stream);
 
 /* act_dtype [n] -> fp16 [n] (saturating); for callers that route elsewhere. */
 int odsd_convert_act_f16(const void *x, int32_t dtype, int64_t n, void *x_f16, void *stream);

@@ -10,10 +10,12 @@ from .w4 import W4ExpertBank, W4ExpertParams, build_table
 from .runner import (MoEOnlyStack, W4MoERunner, expert_forward_with_weights, moe_layer_forward)
 from .placement import (ExpertActivation, LayerExpertActivations, build_layer_activations,
                         build_prefill_placement)
+from .layers import W4MoELayer, W4MoELayerWithWeights, W4Operators
 
 __all__ = [
     "AttentionOutput", "ExpertID", "ExpertPlacement", "LayerOutput", "MoEConfig", "RoutingResult",
     "W4ExpertBank", "W4ExpertParams", "build_table", "MoEOnlyStack", "W4MoERunner",
     "expert_forward_with_weights", "moe_layer_forward", "ops", "workloads",
     "ExpertActivation", "LayerExpertActivations", "build_layer_activations", "build_prefill_placement",
+    "W4MoELayer", "W4MoELayerWithWeights", "W4Operators",
 ]

@@ -93,7 +93,8 @@ static inline size_t odsd_round_up(size_t v, size_t a) { return (v + a - 1) / a 
 // of squares (the router and the fp16 copy then see RMSNorm(x))
 int odsd_launch_router(const odsd_moe_shape *s, const void *x, const void *gate_w, int32_t *idx,
                        float *w, int64_t *idx64, void *x16, void *ws, size_t ws_bytes,
-                       hipStream_t st, const double *norm_ss, const void *norm_w, float eps);
+                       hipStream_t st, const double *norm_ss, const void *norm_w, float eps,
+                       double *logits = nullptr);
 int odsd_launch_dispatch(const odsd_moe_shape *s, const int32_t *idx, int32_t *counts,
                          int32_t *offsets, int32_t *perm, int32_t *inv, int32_t *slot_token,
                          hipStream_t st);

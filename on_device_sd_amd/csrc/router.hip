@@ -219,7 +219,8 @@ __global__ __launch_bounds__(256) void router_topk_kernel(const double *__restri
                                                           int K, int S, int renorm,
                                                           int32_t *__restrict__ idx,
                                                           float *__restrict__ w,
-                                                          int64_t *__restrict__ idx64) {
+                                                          int64_t *__restrict__ idx64,
+                                                          double *__restrict__ logits) {
     const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (t >= T) return;
     const int lane = lane_id();
@@ -249,6 +250,7 @@ __global__ __launch_bounds__(256) void router_topk_kernel(const double *__restri
     for (int v = 0; v < V; ++v) {
         key[v] = order_key(lg[v]);
         if (lane + 64 * v >= E) taken |= 1u << v;
+        else if (logits) logits[(size_t)t * E + lane + 64 * v] = lg[v];
     }
 
     int my_e = 0;          // lane k keeps the k-th winner
@@ -378,7 +380,7 @@ static void launch_partial(const RouterPlan &p, const odsd_moe_shape *s, const v
 
 int odsd_launch_router(const odsd_moe_shape *s, const void *x, const void *gate_w, int32_t *idx, float *w,
                        int64_t *idx64, void *x16, void *ws, size_t ws_bytes, hipStream_t st,
-                       const double *norm_ss, const void *norm_w, float eps) {
+                       const double *norm_ss, const void *norm_w, float eps, double *logits) {
     const int rc = router_check(s);
     if (rc != ODSD_OK) return rc;
     if (s->T == 0) return ODSD_OK;
@@ -404,7 +406,7 @@ int odsd_launch_router(const odsd_moe_shape *s, const void *x, const void *gate_
     const int S_out = p.S % 4 == 0 ? p.S / 4 : p.S;
 #define TOPK_GO(VV)                                                                                   \
     router_topk_kernel<VV><<<(s->T + 3) / 4, 256, 0, st>>>(partial, s->T, s->E, s->K, S_out, s->renorm, \
-                                                            idx, w, idx64)
+                                                            idx, w, idx64, logits)
     if (s->E <= 64) TOPK_GO(1);
     else if (s->E <= 128) TOPK_GO(2);
     else if (s->E <= 256) TOPK_GO(4);
@@ -418,5 +420,14 @@ extern "C" int odsd_router_topk(const odsd_moe_shape *s, const void *x, const vo
                                 int32_t *out_idx, float *out_w, int64_t *out_idx64, void *x_f16,
                                 void *workspace, size_t workspace_bytes, void *stream) {
     return odsd_launch_router(s, x, gate_w, out_idx, out_w, out_idx64, x_f16, workspace, workspace_bytes,
-                              (hipStream_t)stream, nullptr, nullptr, 0.0f);
+                              (hipStream_t)stream, nullptr, nullptr, 0.0f, nullptr);
+}
+
+extern "C" int odsd_router_topk_logits(const odsd_moe_shape *s, const void *x, const void *gate_w,
+                                       int32_t *out_idx, float *out_w, int64_t *out_idx64, void *x_f16,
+                                       double *out_logits, void *workspace, size_t workspace_bytes,
+                                       void *stream) {
+    if (!out_logits) return ODSD_ERR_NULL;
+    return odsd_launch_router(s, x, gate_w, out_idx, out_w, out_idx64, x_f16, workspace, workspace_bytes,
+                              (hipStream_t)stream, nullptr, nullptr, 0.0f, out_logits);
 }

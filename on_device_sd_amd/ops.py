@@ -130,9 +130,9 @@ def to_f16(x: torch.Tensor) -> torch.Tensor:
 # Router / dispatch
 # ------------------------------------------------------------------------------------------
 def router_topk(x: torch.Tensor, gate_weight: torch.Tensor, top_k: int, renorm: bool,
-                want_f16: bool = False, want_int64: bool = False):
+                want_f16: bool = False, want_int64: bool = False, logits_out: Optional[torch.Tensor] = None):
     """x [T,H], gate_weight [E,H] (same dtype) -> (idx int32 [T,K], w float32 [T,K],
-    idx64 or None, x_f16 or None)."""
+    idx64 or None, x_f16 or None).  ``logits_out`` (float64 [T,E], optional) receives the logits."""
     _require_cuda(x, gate_weight)
     lib = _lib.load()
     if gate_weight.dtype != x.dtype:
@@ -150,10 +150,29 @@ def router_topk(x: torch.Tensor, gate_weight: torch.Tensor, top_k: int, renorm: 
     if nbytes == 0:
         raise _lib.OdsdError(f"router: unsupported shape T={T} H={H} E={E} K={top_k}")
     ws = _workspace(nbytes, x.device)
-    _lib.check(lib.odsd_router_topk(C.byref(shape), x.data_ptr(), gate_weight.data_ptr(), idx.data_ptr(),
-                                    w.data_ptr(), _ptr(idx64), _ptr(x16), ws.data_ptr(), ws.numel(),
-                                    _stream()), "odsd_router_topk")
+    if logits_out is not None:
+        if logits_out.dtype != torch.float64 or tuple(logits_out.shape) != (T, E) or \
+                not logits_out.is_contiguous() or not logits_out.is_cuda:
+            raise ValueError("logits_out must be a contiguous float64 [T, E] tensor on the GPU")
+        _lib.check(lib.odsd_router_topk_logits(C.byref(shape), x.data_ptr(), gate_weight.data_ptr(),
+                                               idx.data_ptr(), w.data_ptr(), _ptr(idx64), _ptr(x16),
+                                               logits_out.data_ptr(), ws.data_ptr(), ws.numel(), _stream()),
+                   "odsd_router_topk_logits")
+    else:
+        _lib.check(lib.odsd_router_topk(C.byref(shape), x.data_ptr(), gate_weight.data_ptr(), idx.data_ptr(),
+                                        w.data_ptr(), _ptr(idx64), _ptr(x16), ws.data_ptr(), ws.numel(),
+                                        _stream()), "odsd_router_topk")
     return idx, w, idx64, x16
+
+
+def router_logits(x: torch.Tensor, gate_weight: torch.Tensor) -> torch.Tensor:
+    """scores = F.linear(x, gate_weight) accumulated in fp64: float64 [T, E]
+    (GPUOperators.router, demo/src/operators/gpu_operators.py:48-69)."""
+    x2 = x.reshape(-1, x.shape[-1])
+    out = torch.empty(x2.shape[0], gate_weight.shape[0], dtype=torch.float64, device=x.device)
+    if x2.shape[0]:
+        router_topk(x2, gate_weight, 1, False, logits_out=out)
+    return out
 
 
 @dataclass

@@ -82,8 +82,14 @@ def test_router_indices_bit_exact(dev, T, H, E, K, renorm, dtype):
     g = torch.Generator().manual_seed(T * 7 + E)
     x = torch.randn(T, H, generator=g).to(dtype)
     wg = (torch.randn(E, H, generator=g) * 0.02).to(dtype)
-    idx, w, idx64, x16 = _ops().router_topk(x.to(dev), wg.to(dev), K, renorm, want_f16=True, want_int64=True)
-    idx_o, w_o = orc.route(orc.router_logits(x, wg), K, renorm)
+    logits = torch.empty(T, E, dtype=torch.float64, device=dev)
+    idx, w, idx64, x16 = _ops().router_topk(x.to(dev), wg.to(dev), K, renorm, want_f16=True, want_int64=True,
+                                            logits_out=logits)
+    logits_o = orc.router_logits(x, wg)
+    # fp64 accumulation on both sides: only the summation order differs
+    np.testing.assert_allclose(logits.cpu().numpy(), logits_o.numpy(), rtol=0, atol=1e-12)
+    assert torch.equal(_ops().router_logits(x.to(dev), wg.to(dev)), logits)
+    idx_o, w_o = orc.route(logits_o, K, renorm)
     assert np.array_equal(idx.cpu().numpy(), idx_o)
     assert np.array_equal(idx64.cpu().numpy(), idx_o.astype(np.int64))
     np.testing.assert_allclose(w.cpu().numpy(), w_o, rtol=2e-6, atol=1e-7)
