@@ -11,6 +11,7 @@ from .runner import (MoEOnlyStack, W4MoERunner, expert_forward_with_weights, moe
 from .placement import (ExpertActivation, LayerExpertActivations, build_layer_activations,
                         build_prefill_placement)
 from .layers import W4MoELayer, W4MoELayerWithWeights, W4Operators
+from .cache import LRUStrategy, W4ExpertCache, cache_capacity
 
 __all__ = [
     "AttentionOutput", "ExpertID", "ExpertPlacement", "LayerOutput", "MoEConfig", "RoutingResult",
@@ -18,4 +19,5 @@ __all__ = [
     "expert_forward_with_weights", "moe_layer_forward", "ops", "workloads",
     "ExpertActivation", "LayerExpertActivations", "build_layer_activations", "build_prefill_placement",
     "W4MoELayer", "W4MoELayerWithWeights", "W4Operators",
+    "LRUStrategy", "W4ExpertCache", "cache_capacity",
 ]

@@ -47,6 +47,13 @@ class W4ExpertParams(dict):
         self.bank = bank
         self.expert = expert
         self.ptrs: Tuple[int, int, int, int] = bank.expert_ptrs(expert)
+        # which load of the slot this bundle describes (a cache pool reuses its slots)
+        self.generation: int = bank.generation[expert]
+
+    @property
+    def stale(self) -> bool:
+        """True once the storage behind this bundle has been loaded with other weights."""
+        return self.generation != self.bank.generation[self.expert]
 
 
 class W4ExpertBank:
@@ -62,6 +69,8 @@ class W4ExpertBank:
         self.gu_q, self.gu_sz = mk(self.gu_q_bytes), mk(self.gu_sz_bytes)
         self.dn_q, self.dn_sz = mk(self.dn_q_bytes), mk(self.dn_sz_bytes)
         self.loaded = [False] * E
+        self.generation = [0] * E      # bumped by every load into the slot
+        self.recycles = False          # True for a cache pool, whose slots change owner
         self._bind_storage()
 
     def _bind_storage(self) -> None:
@@ -80,6 +89,8 @@ class W4ExpertBank:
         b.dn_q_bytes, b.dn_sz_bytes = self.dn_q_bytes, self.dn_sz_bytes
         b.gu_q, b.gu_sz, b.dn_q, b.dn_sz = (t.clone() for t in (self.gu_q, self.gu_sz, self.dn_q, self.dn_sz))
         b.loaded = list(self.loaded)
+        b.generation = [0] * self.num_experts
+        b.recycles = False
         b._bind_storage()
         return b
 
@@ -94,7 +105,12 @@ class W4ExpertBank:
         ops.w4_pack_into(*gate, self.gu_q[e], self.gu_sz[e], 2, 0)
         ops.w4_pack_into(*up, self.gu_q[e], self.gu_sz[e], 2, 1)
         ops.w4_pack_into(*down, self.dn_q[e], self.dn_sz[e], 1, 0)
+        self.mark_loaded(e)
+
+    def mark_loaded(self, e: int) -> None:
+        """Slot e holds new weights: bundles handed out before are stale from now on."""
         self.loaded[e] = True
+        self.generation[e] += 1
         self._table = None
 
     def load_expert(self, e: int, gate_w: torch.Tensor, up_w: torch.Tensor, down_w: torch.Tensor,
@@ -142,7 +158,7 @@ class W4ExpertBank:
         if not self.loaded[e]:
             raise KeyError(f"expert {e} has not been loaded")
         p = self._params.get(e)
-        if p is None:
+        if p is None or p.generation != self.generation[e]:
             p = self._params[e] = W4ExpertParams(self, e)
         return p
 
@@ -170,6 +186,8 @@ def build_table(num_experts: int, params: Dict[int, W4ExpertParams],
             p = params[src]
             if not isinstance(p, W4ExpertParams):
                 raise TypeError(f"expert {src}: parameters are not W4 bundles of a W4ExpertBank")
+            if p.stale:
+                raise RuntimeError(f"expert {src}: the bundle is stale (its cache slot holds other weights now)")
             rows.append(p.ptrs)
         else:
             rows.append((0, 0, 0, 0))

@@ -106,3 +106,22 @@ def test_prefill_placement_lookup_order_without_gpu():
     assert {e: p["who"] for e, p in pl.gpu_expert_params.items()} == {3: "shared", 4: "cache", 6: "loader"}
     assert pl.cpu_expert_params == {} and pl.substitution_map == {} and pl.routing_result is rr
     assert ("loader", 3) not in calls and ("loader", 4) not in calls and ("loader", 5) in calls
+
+
+def test_lru_strategy_and_cache_capacity():
+    from on_device_sd_amd.cache import LRUStrategy, cache_capacity
+    ids = [odsd.ExpertID(0, e) for e in range(4)]
+    lru = LRUStrategy()
+    for i in ids[:3]:
+        lru.on_insert(i)
+    lru.on_access(ids[0])
+    assert lru.select_victim(ids[:3], set()) == ids[1]
+    assert lru.select_victim(ids[:3], {ids[1]}) == ids[2]
+    lru.on_evict(ids[1])
+    assert lru.select_victim([ids[0], ids[2]], set()) == ids[2]
+    assert lru.select_victim([ids[3]], set()) == ids[3]          # not tracked: first unpinned
+    assert lru.select_victim(ids[:3], set(ids[:3])) is None
+    # the reference's arithmetic: GB -> MB, then whole experts (expert_cache.py:24-26)
+    assert cache_capacity(1.0, 2.5) == 409 and cache_capacity(0.001, 2.5) == 0
+    cfg = odsd.MoEConfig()
+    assert cache_capacity(16.0, cfg.get_expert_weight_size_bytes() / 2 ** 20) == int(16 * 1024 / (2506752 / 2 ** 20)) == 6853
