@@ -119,8 +119,8 @@ class W4MoERunner:
                tuple(sub.items()) if sub else ())
         hit = self._table_cache.get(key)
         if hit is not None:
-            for p in hit[1]:
-                if p.bank.recycles and p.stale:
+            for p in hit[2]:             # bundles of cache pools only (usually none)
+                if p.stale:
                     raise RuntimeError(f"expert bundle of cache slot {p.expert} is stale: the slot was "
                                        "given to another expert after the placement was built")
             return hit[0]
@@ -135,7 +135,8 @@ class W4MoERunner:
         if len(self._table_cache) > 64:
             self._table_cache.clear()
         tab = build_table(self.config.num_experts, params, sub, self.device)
-        self._table_cache[key] = (tab, list(gpu.values()) + list(cpu.values()))
+        held = list(gpu.values()) + list(cpu.values())
+        self._table_cache[key] = (tab, held, [p for p in held if p.bank.recycles])
         return tab
 
     def _execute_moe_with_placement(self, hidden_states: torch.Tensor, placement: ExpertPlacement,
