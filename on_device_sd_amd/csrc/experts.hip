@@ -77,6 +77,12 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
     const global_char *szp_c = (const global_char *)(MODE == 0 ? trow[1] : trow[3]);
     const global_char *src_c = (const global_char *)p.src;
     const int base = p.offsets[e];
+    // the expert's packed matrix and its (scale, zero) pairs as buffer resources (reads past the
+    // end return zero)
+    const __amdgpu_buffer_rsrc_t rsrc_q = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(uintptr_t)(MODE == 0 ? trow[0] : trow[2]), 0, p.NBLK * p.G * 1024, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_sz = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(uintptr_t)(MODE == 0 ? trow[1] : trow[3]), 0, p.NBLK * p.G * 64, 0x00020000);
 
     const DequantConsts dc = dequant_consts();
     const int tid = threadIdx.x;
@@ -147,17 +153,21 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
         uint32_t wsz[DEPTH][NB];
         uint4_t xd[DIRECT ? DEPTH : 1][4];   // DIRECT: B fragments travel with the ring slot
 
-        // LDS path: the group advances a scalar base and the per-lane offsets never change (the
-        // direct path measured faster with the group folded into the per-lane offset)
+        // LDS path: buffer loads -- the expert's matrix is a buffer resource in scalar registers, the
+        // per-lane byte offset never changes and the group is the scalar offset operand, so a load
+        // costs no vector instruction for its address (the direct path measured faster with plain
+        // global loads and the group folded into the per-lane offset)
         auto load_w = [&](int buf, int g) {
             const uint32_t gc = (uint32_t)min(g, g_last);
-            const global_char *qg = DIRECT ? qp_c : scalar_base(qp_c + (size_t)gc * 1024u);
-            const global_char *sg = DIRECT ? szp_c : scalar_base(szp_c + (size_t)gc * 64u);
-            const uint32_t gq = DIRECT ? gc * 1024u : 0u, gs = DIRECT ? gc * 64u : 0u;
 #pragma unroll
             for (int i = 0; i < NB; ++i) {
-                wq[buf][i] = __builtin_nontemporal_load((const global_u4 *)(qg + (wq_off[i] + gq)));
-                wsz[buf][i] = *(const global_u32 *)(sg + (sz_off[i] + gs));
+                if (DIRECT) {
+                    wq[buf][i] = __builtin_nontemporal_load((const global_u4 *)(qp_c + (wq_off[i] + gc * 1024u)));
+                    wsz[buf][i] = *(const global_u32 *)(szp_c + (sz_off[i] + gc * 64u));
+                } else {
+                    wq[buf][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_q, (int)wq_off[i], (int)(gc * 1024u), 2 /* nt */);
+                    wsz[buf][i] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_sz, (int)sz_off[i], (int)(gc * 64u), 0);
+                }
             }
         };
         // DIRECT: the B fragments of group g (refilled only after the products that read them)
@@ -212,7 +222,9 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
                 // wavefront has passed that step's barrier) and the slot's refill, then the products.
                 // (The compiler cannot see the DMA loads.  Issued after the expansion, the vmcnt
                 // wait it derives for the slot retires exactly the slot and the previous DMA.)
-                const int xb = it & 1;
+                // with an even number of steps per trip the token buffer of a step is known at
+                // compile time (every trip starts on an even step) and becomes an immediate offset
+                const int xb = (DEPTH * RING_TRIPS) % 2 == 0 ? (u & 1) : (it & 1);
                 half8_t bdir[4];
                 if (DIRECT) {
 #pragma unroll
@@ -230,7 +242,7 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
                     for (int i = 0; i < NA; ++i) dequant_tile(dc, wq[d][h + i], wsz[d][h + i], a[i]);
                     if (h + NA >= NB) {
                         __builtin_amdgcn_sched_barrier(0);
-                        if (!DIRECT) dma_x((it + 1) & 1, g + 1);
+                        if (!DIRECT) dma_x(xb ^ 1, g + 1);
                         load_w(d, g + DEPTH);      // ring slot d is free again
                         __builtin_amdgcn_sched_barrier(0);
                     }
