@@ -337,7 +337,11 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
 // out_act = cast(residual + cast(moe)): the reference rounds the MoE output to the
 // activation dtype before the residual add (qwen3_runner.py:295, :226).
 // ---------------------------------------------------------------------------------------------
-template <typename XT, bool YH, bool STATS>
+// KB > 0 (K a multiple of KB, KS == 1): the rows of KB pairs are fetched together -- slot, expert
+// and weight first, then KB independent row loads -- and added in k order; with the generic loop
+// every row load waits for the one before it (its address hangs on a branch), which is what the
+// kernel's time consists of at K = 8.
+template <typename XT, bool YH, bool STATS, int KB>
 __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ y, const int32_t *__restrict__ idx,
                                                       const float *__restrict__ w,
                                                       const int32_t *__restrict__ perm,
@@ -355,6 +359,42 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
         const int c = (blockIdx.x * 256 + threadIdx.x) * 4;
         if (c < H) {
         float4_t acc = {0.f, 0.f, 0.f, 0.f};
+        if (KB > 0) {
+            for (int k0 = 0; k0 < K; k0 += KB) {
+                int slot[KB > 0 ? KB : 1];
+                float wk[KB > 0 ? KB : 1];
+                bool ok[KB > 0 ? KB : 1];
+#pragma unroll
+                for (int u = 0; u < KB; ++u) {
+                    const int pr = t * K + k0 + u;
+                    const int sl = perm[pr];
+                    const int e = idx[pr];
+                    wk[u] = w[pr];
+                    const bool in_range = sl >= 0 && e >= 0 && e < E;
+                    ok[u] = in_range && table[(size_t)(in_range ? e : 0) * ODSD_TABLE_COLS] != 0;
+                    slot[u] = ok[u] ? sl : 0;      // a row that exists; its values are discarded below
+                }
+                float4_t v[KB > 0 ? KB : 1];
+#pragma unroll
+                for (int u = 0; u < KB; ++u) {
+                    if (YH) {
+                        const half4_t hv = *(const half4_t *)((const half_t *)y + (size_t)slot[u] * H + c);
+                        v[u] = float4_t{(float)hv.x, (float)hv.y, (float)hv.z, (float)hv.w};
+                    } else {
+                        v[u] = *(const float4_t *)(y + (size_t)slot[u] * H + c);
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < KB; ++u) {
+                    if (ok[u]) {
+                        acc.x = fmaf(wk[u], v[u].x, acc.x);
+                        acc.y = fmaf(wk[u], v[u].y, acc.y);
+                        acc.z = fmaf(wk[u], v[u].z, acc.z);
+                        acc.w = fmaf(wk[u], v[u].w, acc.w);
+                    }
+                }
+            }
+        } else {
         for (int k = 0; k < K; ++k) {
             const int pr = t * K + k;
             const int slot = perm[pr];
@@ -374,6 +414,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
             acc.y = fmaf(wk, v.y, acc.y);
             acc.z = fmaf(wk, v.z, acc.z);
             acc.w = fmaf(wk, v.w, acc.w);
+        }
         }
         const size_t o = (size_t)t * H + c;
         float res[4] = {0.f, 0.f, 0.f, 0.f};
@@ -606,10 +647,18 @@ static int launch_combine(const odsd_moe_shape *s, const void *y_, const int32_t
     const ExpertsPlan pl = experts_plan(s);
     const int P = s->T * s->K;
     const dim3 grid((s->H / 4 + 255) / 256, s->T);
+    const bool batched = pl.KS == 1 && s->K % 4 == 0;      // rows of 4 pairs fetched together (8: no faster)
 #define COMBINE_GO(XT, YH, ST)                                                                          \
-    combine_kernel<XT, YH, ST><<<grid, 256, 0, st>>>(y, idx, w, perm, table, (const XT *)residual,     \
-                                                     out_f32, (XT *)out_act, row_ss, s->T, s->H, s->K, \
-                                                     s->E, pl.KS, P)
+    do {                                                                                                \
+        if (batched)                                                                                    \
+            combine_kernel<XT, YH, ST, 4><<<grid, 256, 0, st>>>(y, idx, w, perm, table, (const XT *)residual, \
+                                                                out_f32, (XT *)out_act, row_ss, s->T, s->H,   \
+                                                                s->K, s->E, pl.KS, P);                        \
+        else                                                                                            \
+            combine_kernel<XT, YH, ST, 0><<<grid, 256, 0, st>>>(y, idx, w, perm, table, (const XT *)residual, \
+                                                                out_f32, (XT *)out_act, row_ss, s->T, s->H,   \
+                                                                s->K, s->E, pl.KS, P);                        \
+    } while (0)
 #define COMBINE_Y(XT, ST)                          \
     do {                                           \
         if (pl.y_f16) COMBINE_GO(XT, true, ST);    \
