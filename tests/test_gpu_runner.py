@@ -106,6 +106,23 @@ def test_substitution_uses_substitute_params(runner, dev):
     assert out.abs().sum() > 0
 
 
+def test_four_pairs_per_token_with_absent_and_repeated_experts(runner, dev):
+    """K = 4 takes the combine's batched row fetch; pairs of an expert that is not placed are
+    skipped there without their rows being used."""
+    import on_device_sd_amd as odsd
+    hidden = _hidden(dev, 3, H, seed=8)
+    idx = torch.tensor([[0, 1, 2, 3], [3, 2, 1, 0], [1, 1, 2, 2]], device=dev)
+    g = torch.Generator().manual_seed(9)
+    scores = torch.rand(3, 4, generator=g).to(dev)
+    params = {e: p for e, p in runner.banks[0].all_expert_params().items() if e != 2}
+    placement = odsd.ExpertPlacement(gpu_expert_params=params, cpu_expert_params={},
+                                     routing_result=_routing(0, idx, scores))
+    out = runner._execute_moe_with_placement(hidden, placement)
+    ref = orc.moe_forward(hidden.cpu(), idx.cpu().numpy(), scores.cpu().numpy(),
+                          {e: x for e, x in runner.oracle_experts[0].items() if e != 2})
+    check_output(out, ref)
+
+
 def test_empty_routing_gives_zero_moe_contribution(runner, dev):
     import on_device_sd_amd as odsd
     hidden = _hidden(dev, 2, H)
