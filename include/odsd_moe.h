@@ -20,6 +20,7 @@
  * potatoZhx/on_device_sd tree):
  *   odsd_router_topk   Qwen3MoEGate.forward                    demo/src/layers/moe_layer.py:25-60
  *   odsd_router_topk_logits  + GPUOperators.router            demo/src/operators/gpu_operators.py:48-69
+ *   odsd_route_dispatch      Qwen3ModelRunner.route_experts    demo/src/model/qwen3_runner.py:86-119
  *                      Qwen3ModelRunner.route_experts          demo/src/model/qwen3_runner.py:86-119
  *                      GPUOperators.router                     demo/src/operators/gpu_operators.py:48-69
  *   odsd_dispatch      mask / torch.where per expert           demo/src/model/qwen3_runner.py:303-314
@@ -130,6 +131,14 @@ int odsd_router_topk_logits(const odsd_moe_shape *s, const void *x, const void *
 
 /* act_dtype [n] -> fp16 [n] (saturating); for callers that route elsewhere. */
 int odsd_convert_act_f16(const void *x, int32_t dtype, int64_t n, void *x_f16, void *stream);
+
+/* Router and dispatch in one call: what route_experts does before the host reads the activated
+ * set (demo/src/model/qwen3_runner.py:86-119 followed by the per-expert masks of :303-314).
+ * Outputs as odsd_router_topk and odsd_dispatch below. */
+int odsd_route_dispatch(const odsd_moe_shape *s, const void *x, const void *gate_w,
+                        int32_t *out_idx, float *out_w, int64_t *out_idx64, void *x_f16,
+                        int32_t *counts, int32_t *offsets, int32_t *perm, int32_t *inv,
+                        int32_t *slot_token, void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---- Dispatch ----------------------------------------------------------------------- */
 /* Stable counting sort of the P pairs by expert id.

@@ -88,10 +88,10 @@ extern "C" int odsd_moe_forward(const odsd_moe_shape *s, const void *x, const vo
         if (rc != ODSD_OK) return rc;
         xin = ws + l.xn;
     }
+    const OdsdDispatchOut disp{counts, offsets, perm, inv, slot_token};
     int rc = odsd_launch_router(s, xin, gate_w, idx, w, nullptr, x16, ws + l.router,
-                                l.xn - l.router, st, fold ? row_sumsq_in : nullptr, norm_weight, eps);
-    if (rc != ODSD_OK) return rc;
-    rc = odsd_launch_dispatch(s, idx, counts, offsets, perm, inv, slot_token, st);
+                                l.xn - l.router, st, fold ? row_sumsq_in : nullptr, norm_weight, eps,
+                                nullptr, &disp);
     if (rc != ODSD_OK) return rc;
     return odsd_launch_experts(s, x16, table, idx, w, counts, offsets, perm, slot_token,
                                add_residual ? x : nullptr, out_f32, out_act, ws + l.experts,

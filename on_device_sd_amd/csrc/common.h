@@ -91,10 +91,15 @@ static inline size_t odsd_round_up(size_t v, size_t a) { return (v + a - 1) / a 
 // kernels implemented in the other translation units (host launchers)
 // norm_ss/norm_w/eps: when norm_ss is given, x is RMS-normalised on the fly from the per-row sums
 // of squares (the router and the fp16 copy then see RMSNorm(x))
+// dispatch arrays a router launch may fill as well (all five or none)
+struct OdsdDispatchOut {
+    int32_t *counts, *offsets, *perm, *inv, *slot_token;
+};
+// router (+ dispatch when `disp` is given)
 int odsd_launch_router(const odsd_moe_shape *s, const void *x, const void *gate_w, int32_t *idx,
                        float *w, int64_t *idx64, void *x16, void *ws, size_t ws_bytes,
                        hipStream_t st, const double *norm_ss, const void *norm_w, float eps,
-                       double *logits = nullptr);
+                       double *logits = nullptr, const OdsdDispatchOut *disp = nullptr);
 int odsd_launch_dispatch(const odsd_moe_shape *s, const int32_t *idx, int32_t *counts,
                          int32_t *offsets, int32_t *perm, int32_t *inv, int32_t *slot_token,
                          hipStream_t st);

@@ -380,9 +380,12 @@ static void launch_partial(const RouterPlan &p, const odsd_moe_shape *s, const v
 
 int odsd_launch_router(const odsd_moe_shape *s, const void *x, const void *gate_w, int32_t *idx, float *w,
                        int64_t *idx64, void *x16, void *ws, size_t ws_bytes, hipStream_t st,
-                       const double *norm_ss, const void *norm_w, float eps, double *logits) {
+                       const double *norm_ss, const void *norm_w, float eps, double *logits,
+                       const OdsdDispatchOut *disp) {
     const int rc = router_check(s);
     if (rc != ODSD_OK) return rc;
+    if (disp && (!disp->counts || !disp->offsets || !disp->perm || !disp->inv || !disp->slot_token))
+        return ODSD_ERR_NULL;
     if (s->T == 0) return ODSD_OK;
     if (!x || !gate_w || !idx || !w || !ws) return ODSD_ERR_NULL;
     if (norm_ss && (!norm_w || !odsd_aligned16(norm_w))) return norm_w ? ODSD_ERR_ALIGN : ODSD_ERR_NULL;
@@ -413,6 +416,7 @@ int odsd_launch_router(const odsd_moe_shape *s, const void *x, const void *gate_
     else TOPK_GO(8);
 #undef TOPK_GO
     ODSD_CHECK_LAUNCH();
+    if (disp) return odsd_launch_dispatch(s, idx, disp->counts, disp->offsets, disp->perm, disp->inv, disp->slot_token, st);
     return ODSD_OK;
 }
 
@@ -420,7 +424,16 @@ extern "C" int odsd_router_topk(const odsd_moe_shape *s, const void *x, const vo
                                 int32_t *out_idx, float *out_w, int64_t *out_idx64, void *x_f16,
                                 void *workspace, size_t workspace_bytes, void *stream) {
     return odsd_launch_router(s, x, gate_w, out_idx, out_w, out_idx64, x_f16, workspace, workspace_bytes,
-                              (hipStream_t)stream, nullptr, nullptr, 0.0f, nullptr);
+                              (hipStream_t)stream, nullptr, nullptr, 0.0f, nullptr, nullptr);
+}
+
+extern "C" int odsd_route_dispatch(const odsd_moe_shape *s, const void *x, const void *gate_w,
+                                   int32_t *out_idx, float *out_w, int64_t *out_idx64, void *x_f16,
+                                   int32_t *counts, int32_t *offsets, int32_t *perm, int32_t *inv,
+                                   int32_t *slot_token, void *workspace, size_t workspace_bytes, void *stream) {
+    const OdsdDispatchOut d{counts, offsets, perm, inv, slot_token};
+    return odsd_launch_router(s, x, gate_w, out_idx, out_w, out_idx64, x_f16, workspace, workspace_bytes,
+                              (hipStream_t)stream, nullptr, nullptr, 0.0f, nullptr, &d);
 }
 
 extern "C" int odsd_router_topk_logits(const odsd_moe_shape *s, const void *x, const void *gate_w,
@@ -429,5 +442,5 @@ extern "C" int odsd_router_topk_logits(const odsd_moe_shape *s, const void *x, c
                                        void *stream) {
     if (!out_logits) return ODSD_ERR_NULL;
     return odsd_launch_router(s, x, gate_w, out_idx, out_w, out_idx64, x_f16, workspace, workspace_bytes,
-                              (hipStream_t)stream, nullptr, nullptr, 0.0f, out_logits);
+                              (hipStream_t)stream, nullptr, nullptr, 0.0f, out_logits, nullptr);
 }

@@ -212,6 +212,47 @@ def dispatch(idx: torch.Tensor, num_experts: int, idx32_keep: bool = False) -> D
     return d
 
 
+def route_dispatch(x: torch.Tensor, gate_weight: torch.Tensor, top_k: int, renorm: bool,
+                   want_f16: bool = True, want_int64: bool = True):
+    """Router, top-k and dispatch in one library call.
+    Returns (idx int32 [T,K], w float32 [T,K], idx64 or None, x_f16 or None, Dispatch)."""
+    _require_cuda(x, gate_weight)
+    lib = _lib.load()
+    if gate_weight.dtype != x.dtype:
+        gate_weight = gate_weight.to(x.dtype)
+    x = x.contiguous()
+    gate_weight = gate_weight.contiguous()
+    T, H = x.shape
+    E = gate_weight.shape[0]
+    dev = x.device
+    shape = make_shape(T, H, E, top_k, 128, renorm, x.dtype)
+    P = T * top_k
+    # one int32 allocation: idx [T,K], counts [E], offsets [E+1], perm / inv / slot_token [P]
+    p_pad, e_pad, e1_pad = (P + 3) & ~3, (E + 3) & ~3, (E + 4) & ~3
+    buf = torch.empty(4 * p_pad + e_pad + e1_pad, dtype=torch.int32, device=dev)
+    o = [0, p_pad, p_pad + e_pad, p_pad + e_pad + e1_pad, 2 * p_pad + e_pad + e1_pad, 3 * p_pad + e_pad + e1_pad]
+    idx = buf[o[0]:o[0] + P].view(T, top_k)
+    d = Dispatch(buf[o[1]:o[1] + E], buf[o[2]:o[2] + E + 1], buf[o[3]:o[3] + P], buf[o[4]:o[4] + P],
+                 buf[o[5]:o[5] + P], idx)
+    w = torch.empty(T, top_k, dtype=torch.float32, device=dev)
+    idx64 = torch.empty(T, top_k, dtype=torch.int64, device=dev) if want_int64 else None
+    x16 = torch.empty(T, H, dtype=torch.float16, device=dev) if want_f16 else None
+    if T == 0:
+        d.counts.zero_()
+        d.offsets.zero_()
+        return idx, w, idx64, x16, d
+    nbytes = lib.odsd_router_workspace_bytes(C.byref(shape))
+    if nbytes == 0:
+        raise _lib.OdsdError(f"router: unsupported shape T={T} H={H} E={E} K={top_k}")
+    ws = _workspace(nbytes, dev)
+    _lib.check(lib.odsd_route_dispatch(C.byref(shape), x.data_ptr(), gate_weight.data_ptr(), idx.data_ptr(),
+                                       w.data_ptr(), _ptr(idx64), _ptr(x16), d.counts.data_ptr(),
+                                       d.offsets.data_ptr(), d.perm.data_ptr(), d.inv.data_ptr(),
+                                       d.slot_token.data_ptr(), ws.data_ptr(), ws.numel(), _stream()),
+               "odsd_route_dispatch")
+    return idx, w, idx64, x16, d
+
+
 # ------------------------------------------------------------------------------------------
 # Experts + combine, whole block
 # ------------------------------------------------------------------------------------------

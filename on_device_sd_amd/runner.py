@@ -64,10 +64,8 @@ class W4MoERunner:
     def route_experts(self, layer_idx: int, hidden_states: torch.Tensor) -> RoutingResult:
         cfg = self.config
         flat = hidden_states.reshape(-1, hidden_states.shape[-1])
-        idx32, w, idx64, x16 = ops.router_topk(flat, self.gate_weights[layer_idx],
-                                               cfg.num_experts_per_token, cfg.norm_topk_prob,
-                                               want_f16=True, want_int64=True)
-        disp = ops.dispatch(idx32, cfg.num_experts, idx32_keep=True)
+        _, w, idx64, x16, disp = ops.route_dispatch(flat, self.gate_weights[layer_idx],
+                                                    cfg.num_experts_per_token, cfg.norm_topk_prob)
         # the engine reads the activated set on the host between routing and execution
         # (qwen3_runner.py:110-112): one asynchronous copy of the E counts into pinned memory,
         # and a wait for that copy alone

@@ -56,6 +56,9 @@ def test_argument_checks_need_no_gpu():
     assert lib.odsd_add_rmsnorm(None, None, None, 1, 4, 128, 1e-6, None, None, None) == 1
     assert lib.odsd_add_rmsnorm(1 << 20, 1 << 20, 1 << 20, 7, 4, 128, 1e-6, 1 << 20, 1 << 20, None) == 7
     assert lib.odsd_router_topk(C.byref(ok), None, None, None, None, None, None, None, 0, None) == 1
+    # the combined call needs all five dispatch arrays
+    assert lib.odsd_route_dispatch(C.byref(ok), 1 << 20, 1 << 20, 1 << 20, 1 << 20, None, None, 1 << 20, None,
+                                   1 << 20, 1 << 20, 1 << 20, 1 << 20, 1 << 30, None) == 1
     # the logits form needs its extra output
     assert lib.odsd_router_topk_logits(C.byref(ok), 1 << 20, 1 << 20, 1 << 20, 1 << 20, None, None, None,
                                        1 << 20, 1 << 30, None) == 1

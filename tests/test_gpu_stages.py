@@ -112,6 +112,39 @@ def test_router_ties_lower_index_first(dev):
     idx, _, _, _ = _ops().router_topk(torch.zeros(3, 256, dtype=torch.bfloat16, device=dev),
                                       (torch.randn(16, 256, generator=g) * 0.02).to(torch.bfloat16).to(dev), 4, False)
     assert np.array_equal(idx.cpu().numpy(), np.tile(np.arange(4, dtype=np.int32), (3, 1)))
+    # 8 identical gate rows, 5 tokens
+    idx, w, _, _ = _ops().router_topk(x[:5].to(dev), row.repeat(8, 1).to(dev), 3, True)
+    assert np.array_equal(idx.cpu().numpy(), np.tile(np.arange(3, dtype=np.int32), (5, 1)))
+    np.testing.assert_allclose(w.cpu().numpy(), 1.0 / 3.0, rtol=1e-6)
+
+
+@pytest.mark.parametrize("T,H,E,K,renorm,dtype", [
+    (5, 4096, 8, 2, False, torch.bfloat16),
+    (8, 256, 8, 8, True, torch.float32),        # K == E
+    (3, 384, 5, 3, True, torch.bfloat16),       # odd number of column groups
+    (1, 128, 1, 1, False, torch.float32),
+    (40, 512, 60, 6, False, torch.bfloat16),
+])
+def test_route_dispatch_one_call(dev, T, H, E, K, renorm, dtype):
+    print("route_dispatch", T, H, E, K, renorm, dtype, flush=True)
+    g = torch.Generator().manual_seed(T * 11 + E)
+    x = torch.randn(T, H, generator=g).to(dtype)
+    wg = (torch.randn(E, H, generator=g) * 0.05).to(dtype)
+    idx, w, idx64, x16, d = _ops().route_dispatch(x.to(dev), wg.to(dev), K, renorm)
+    idx_o, w_o = orc.route(orc.router_logits(x, wg), K, renorm)
+    assert np.array_equal(idx.cpu().numpy(), idx_o) and np.array_equal(idx64.cpu().numpy(), idx_o.astype(np.int64))
+    np.testing.assert_allclose(w.cpu().numpy(), w_o, rtol=2e-6, atol=1e-7)
+    assert torch.equal(x16.cpu(), x.to(torch.float16))
+    c, o, perm, inv = orc.dispatch(idx_o, E)
+    assert np.array_equal(d.counts.cpu().numpy(), c) and np.array_equal(d.offsets.cpu().numpy(), o)
+    assert np.array_equal(d.perm.cpu().numpy(), perm) and np.array_equal(d.inv.cpu().numpy(), inv)
+    assert np.array_equal(d.slot_token.cpu().numpy(), inv // K)
+    # the separate calls give the same bits
+    idx2, w2, _, _ = _ops().router_topk(x.to(dev), wg.to(dev), K, renorm)
+    assert torch.equal(idx2, idx) and torch.equal(w2, w)
+    logits = torch.empty(T, E, dtype=torch.float64, device=dev)
+    _ops().router_topk(x.to(dev), wg.to(dev), K, renorm, logits_out=logits)
+    np.testing.assert_allclose(logits.cpu().numpy(), orc.router_logits(x, wg).numpy(), rtol=0, atol=1e-12)
 
 
 @pytest.mark.parametrize("T,K,E", [(32, 2, 8), (5, 2, 8), (160, 2, 8), (64, 8, 128), (256, 8, 128),
