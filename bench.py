@@ -64,6 +64,25 @@ def _event_ms(fn, n):
     return sum(ts) / len(ts), ts[len(ts) // 2], ts[0]
 
 
+def _event_ms_sequence(stages, n):
+    """Average / median / minimum duration of every stage of a sequence that is launched n times
+    back to back, with an event between consecutive stages (on the launch stream)."""
+    import torch
+    ns = len(stages)
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(ns + 1)] for _ in range(n)]
+    for i in range(n):
+        evs[i][0].record()
+        for k, fn in enumerate(stages):
+            fn(i)
+            evs[i][k + 1].record()
+    torch.cuda.synchronize()
+    out = []
+    for k in range(ns):
+        ts = sorted(evs[i][k].elapsed_time(evs[i][k + 1]) for i in range(n))
+        out.append((sum(ts) / len(ts), ts[len(ts) // 2], ts[0]))
+    return out
+
+
 def bench_layer(wl, dev, steps, warmup, with_cpu):
     import torch
     from on_device_sd_amd import ops
@@ -97,12 +116,17 @@ def bench_layer(wl, dev, steps, warmup, with_cpu):
     n = max(steps, 10)
     for i in range(3):
         st.gate_up(x16, tables[i % n_rep], disp); st.down(tables[i % n_rep], disp)
-    k_gu = _event_ms(lambda i: st.gate_up(x16, tables[i % n_rep], disp), n)
-    k_dn = _event_ms(lambda i: st.down(tables[i % n_rep], disp), n)
-    k_cb = _event_ms(lambda i: st.combine(idx, w, disp, tables[0], out_f32=out32), n)
-    k_rt = _event_ms(lambda i: ops.router_topk(x, gate, wl.K, wl.renorm, want_f16=True), n)
-    k_dp = _event_ms(lambda i: ops.dispatch(idx, wl.E), n)
-
+    # every stage bracketed by its own events INSIDE the sequence of a whole step (router ->
+    # dispatch -> gate_up -> down -> combine), so that each kernel is timed under the clocks and
+    # cache state it sees in the timed region, not in a loop of its own
+    stages = [
+        lambda i: ops.router_topk(x, gate, wl.K, wl.renorm, want_f16=True),
+        lambda i: ops.dispatch(idx, wl.E),
+        lambda i: st.gate_up(x16, tables[i % n_rep], disp),
+        lambda i: st.down(tables[i % n_rep], disp),
+        lambda i: st.combine(idx, w, disp, tables[0], out_f32=out32),
+    ]
+    k_rt, k_dp, k_gu, k_dn, k_cb = _event_ms_sequence(stages, n)
     # the two-call path of the reference engine loops: route_experts, the host reads the
     # activated set, forward_moe (reported beside the whole-block call, never as `value`)
     import on_device_sd_amd as odsd
