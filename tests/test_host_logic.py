@@ -125,3 +125,10 @@ def test_lru_strategy_and_cache_capacity():
     assert cache_capacity(1.0, 2.5) == 409 and cache_capacity(0.001, 2.5) == 0
     cfg = odsd.MoEConfig()
     assert cache_capacity(16.0, cfg.get_expert_weight_size_bytes() / 2 ** 20) == int(16 * 1024 / (2506752 / 2 ** 20)) == 6853
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess, sys, os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0 and "one GPU" in r.stderr and r.stdout.strip() == ""
