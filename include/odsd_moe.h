@@ -54,7 +54,9 @@ typedef enum odsd_status {
     ODSD_ERR_ALIGN = 4,       /* a pointer is not 16-byte aligned                        */
     ODSD_ERR_WORKSPACE = 5,   /* workspace smaller than the *_workspace_bytes() answer   */
     ODSD_ERR_LAUNCH = 6,      /* the HIP runtime refused a launch                        */
-    ODSD_ERR_DTYPE = 7        /* unknown dtype code                                      */
+    ODSD_ERR_DTYPE = 7,       /* unknown dtype code                                      */
+    ODSD_ERR_SCRATCH = 8      /* odsd_moe_forward_static: the shape needs more than
+                                 ODSD_STATIC_SCRATCH_BYTES of scratch memory             */
 } odsd_status;
 
 enum { ODSD_DT_F32 = 0, ODSD_DT_BF16 = 1 };
@@ -196,6 +198,22 @@ int odsd_moe_forward(const odsd_moe_shape *s, const void *x, const void *norm_we
                      int32_t *out_offsets, int32_t *out_perm,
                      const double *row_sumsq_in, double *row_sumsq_out,
                      void *workspace, size_t workspace_bytes, void *stream);
+
+/* odsd_moe_forward without a workspace argument and without any allocation, for callers that
+ * cannot call hipMalloc: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid it.  It has no counterpart in the reference.  The workspace is a device array inside
+ * the library (ODSD_STATIC_SCRATCH_BYTES per GPU the library runs on, held until the process
+ * ends).  A shape whose odsd_moe_workspace_bytes() exceeds that size is refused with
+ * ODSD_ERR_SCRATCH.  All calls on one GPU share the one array: calls that overlap on a GPU
+ * (two streams, two threads) race; run them one after the other.  Arguments and results are
+ * those of odsd_moe_forward. */
+#define ODSD_STATIC_SCRATCH_BYTES (64u << 20)
+int odsd_moe_forward_static(const odsd_moe_shape *s, const void *x, const void *norm_weight,
+                            float eps, const void *gate_w, const uint64_t *table,
+                            int32_t add_residual, float *out_f32, void *out_act,
+                            int32_t *out_idx, float *out_w, int32_t *out_counts,
+                            int32_t *out_offsets, int32_t *out_perm,
+                            const double *row_sumsq_in, double *row_sumsq_out, void *stream);
 
 #ifdef __cplusplus
 }

@@ -53,7 +53,11 @@ SIGNATURES = {
     "odsd_moe_workspace_bytes": (C.c_size_t, [_SP]),
     "odsd_moe_forward": (C.c_int, [_SP, _P, _P, C.c_float, _P, _P, C.c_int32, _P, _P, _P, _P, _P, _P,
                                    _P, _P, _P, _P, C.c_size_t, _P]),
+    "odsd_moe_forward_static": (C.c_int, [_SP, _P, _P, C.c_float, _P, _P, C.c_int32, _P, _P, _P, _P, _P,
+                                          _P, _P, _P, _P, _P]),
 }
+
+STATIC_SCRATCH_BYTES = 64 << 20        # ODSD_STATIC_SCRATCH_BYTES
 
 _lib: Optional[C.CDLL] = None
 

@@ -6,6 +6,8 @@
 // in between.
 #include "common.h"
 
+#include <mutex>
+
 extern "C" int odsd_version(void) { return ODSD_VERSION; }
 
 extern "C" const char *odsd_status_string(int status) {
@@ -18,6 +20,7 @@ extern "C" const char *odsd_status_string(int status) {
         case ODSD_ERR_WORKSPACE: return "workspace too small";
         case ODSD_ERR_LAUNCH: return "HIP launch failed";
         case ODSD_ERR_DTYPE: return "unknown dtype code";
+        case ODSD_ERR_SCRATCH: return "the call needs more scratch memory than the library's static array holds";
         default: return "unknown status";
     }
 }
@@ -53,12 +56,14 @@ extern "C" size_t odsd_moe_workspace_bytes(const odsd_moe_shape *s) {
     return moe_layout(s).total;
 }
 
-extern "C" int odsd_moe_forward(const odsd_moe_shape *s, const void *x, const void *norm_weight, float eps,
-                                const void *gate_w, const uint64_t *table, int32_t add_residual,
-                                float *out_f32, void *out_act, int32_t *out_idx, float *out_w,
-                                int32_t *out_counts, int32_t *out_offsets, int32_t *out_perm,
-                                const double *row_sumsq_in, double *row_sumsq_out,
-                                void *workspace, size_t workspace_bytes, void *stream) {
+// One whole block.  `events` (optional, ODSD_N_STAGES + 1 hipEvent_t handles): event 0 is recorded
+// before the first launch and event k + 1 after the launches of stage k .
+static int moe_forward_impl(const odsd_moe_shape *s, const void *x, const void *norm_weight, float eps,
+                            const void *gate_w, const uint64_t *table, int32_t add_residual,
+                            float *out_f32, void *out_act, int32_t *out_idx, float *out_w,
+                            int32_t *out_counts, int32_t *out_offsets, int32_t *out_perm,
+                            const double *row_sumsq_in, double *row_sumsq_out,
+                            void *workspace, size_t workspace_bytes, void *stream, void *const *events) {
     if (!s) return ODSD_ERR_NULL;
     const size_t need = odsd_moe_workspace_bytes(s);
     if (need == 0) return ODSD_ERR_SHAPE;
@@ -77,6 +82,12 @@ extern "C" int odsd_moe_forward(const odsd_moe_shape *s, const void *x, const vo
     int32_t *inv = (int32_t *)(ws + l.inv);
     int32_t *slot_token = (int32_t *)(ws + l.slot_token);
     void *x16 = ws + l.x16;
+    int n_ev = 0;
+#define ODSD_STAGE_DONE()                                                                        \
+    do {                                                                                         \
+        if (events && hipEventRecord((hipEvent_t)events[n_ev++], st) != hipSuccess) return ODSD_ERR_LAUNCH; \
+    } while (0)
+    ODSD_STAGE_DONE();
 
     // RMSNorm: with the row statistics at hand (left by the previous block's combine) the router
     // kernel normalises on the fly; otherwise the stand-alone kernel runs first
@@ -88,12 +99,76 @@ extern "C" int odsd_moe_forward(const odsd_moe_shape *s, const void *x, const vo
         if (rc != ODSD_OK) return rc;
         xin = ws + l.xn;
     }
-    const OdsdDispatchOut disp{counts, offsets, perm, inv, slot_token};
+    ODSD_STAGE_DONE();   // ODSD_STAGE_NORM
     int rc = odsd_launch_router(s, xin, gate_w, idx, w, nullptr, x16, ws + l.router,
                                 l.xn - l.router, st, fold ? row_sumsq_in : nullptr, norm_weight, eps,
-                                nullptr, &disp);
+                                nullptr, nullptr);
     if (rc != ODSD_OK) return rc;
+    ODSD_STAGE_DONE();   // ODSD_STAGE_ROUTER
+    rc = odsd_launch_dispatch(s, idx, counts, offsets, perm, inv, slot_token, st);
+    if (rc != ODSD_OK) return rc;
+    ODSD_STAGE_DONE();   // ODSD_STAGE_DISPATCH
     return odsd_launch_experts(s, x16, table, idx, w, counts, offsets, perm, slot_token,
                                add_residual ? x : nullptr, out_f32, out_act, ws + l.experts,
-                               l.total - l.experts, st, row_sumsq_out);
+                               l.total - l.experts, st, row_sumsq_out, events ? events + n_ev : nullptr);
+#undef ODSD_STAGE_DONE
+}
+
+extern "C" int odsd_moe_forward(const odsd_moe_shape *s, const void *x, const void *norm_weight, float eps,
+                                const void *gate_w, const uint64_t *table, int32_t add_residual,
+                                float *out_f32, void *out_act, int32_t *out_idx, float *out_w,
+                                int32_t *out_counts, int32_t *out_offsets, int32_t *out_perm,
+                                const double *row_sumsq_in, double *row_sumsq_out,
+                                void *workspace, size_t workspace_bytes, void *stream) {
+    return moe_forward_impl(s, x, norm_weight, eps, gate_w, table, add_residual, out_f32, out_act, out_idx,
+                            out_w, out_counts, out_offsets, out_perm, row_sumsq_in, row_sumsq_out,
+                            workspace, workspace_bytes, stream, nullptr);
+}
+
+// ---- the whole block for callers that cannot allocate -------------------------------------------
+// The workspace of odsd_moe_forward lives in a device array of this library instead of coming from
+// the caller.  Each GPU holds its own copy of the array at its own address; the address is looked
+// up once per device (with that device current) and used from then on -- the array's name itself
+// means nothing to host code.
+static __device__ __align__(256) unsigned char scratch[ODSD_STATIC_SCRATCH_BYTES];
+
+#define ODSD_MAX_DEVICES 64
+static std::mutex scratch_mutex;
+static void *scratch_ptr[ODSD_MAX_DEVICES];   // per device, filled on the first call on that device
+
+static int scratch_for_current_device(void **out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= ODSD_MAX_DEVICES) return ODSD_ERR_LAUNCH;
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (!scratch_ptr[dev]) {
+        void *p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) {
+            (void)hipGetLastError();
+            return ODSD_ERR_LAUNCH;
+        }
+        scratch_ptr[dev] = p;
+    }
+    *out = scratch_ptr[dev];
+    return ODSD_OK;
+}
+
+extern "C" int odsd_moe_forward_static(const odsd_moe_shape *s, const void *x, const void *norm_weight,
+                                       float eps, const void *gate_w, const uint64_t *table,
+                                       int32_t add_residual, float *out_f32, void *out_act,
+                                       int32_t *out_idx, float *out_w, int32_t *out_counts,
+                                       int32_t *out_offsets, int32_t *out_perm,
+                                       const double *row_sumsq_in, double *row_sumsq_out, void *stream) {
+    if (!s) return ODSD_ERR_NULL;
+    const size_t need = odsd_moe_workspace_bytes(s);
+    if (need == 0) return ODSD_ERR_SHAPE;
+    if (need > (size_t)ODSD_STATIC_SCRATCH_BYTES) return ODSD_ERR_SCRATCH;
+    if (s->T == 0) return ODSD_OK;
+    void *ws = nullptr;
+    const int rc = scratch_for_current_device(&ws);
+    if (rc != ODSD_OK) return rc;
+    // every kernel of the block writes what it later reads, so nothing in the array has to start at
+    // zero and the previous call's contents are simply overwritten
+    return moe_forward_impl(s, x, norm_weight, eps, gate_w, table, add_residual, out_f32, out_act, out_idx,
+                            out_w, out_counts, out_offsets, out_perm, row_sumsq_in, row_sumsq_out, ws,
+                            (size_t)ODSD_STATIC_SCRATCH_BYTES, stream, nullptr);
 }

@@ -107,4 +107,5 @@ int odsd_launch_experts(const odsd_moe_shape *s, const void *x16, const uint64_t
                         const int32_t *idx, const float *w, const int32_t *counts,
                         const int32_t *offsets, const int32_t *perm, const int32_t *slot_token,
                         const void *residual, float *out_f32, void *out_act, void *ws,
-                        size_t ws_bytes, hipStream_t st, double *row_ss);
+                        size_t ws_bytes, hipStream_t st, double *row_ss,
+                        void *const *events = nullptr);   // 3 events: after gate_up, down, combine

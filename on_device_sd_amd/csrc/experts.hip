@@ -686,7 +686,7 @@ extern "C" int odsd_combine(const odsd_moe_shape *s, const void *y, const int32_
 int odsd_launch_experts(const odsd_moe_shape *s, const void *x16, const uint64_t *table, const int32_t *idx,
                         const float *w, const int32_t *counts, const int32_t *offsets, const int32_t *perm,
                         const int32_t *slot_token, const void *residual, float *out_f32, void *out_act,
-                        void *ws, size_t ws_bytes, hipStream_t st, double *row_ss) {
+                        void *ws, size_t ws_bytes, hipStream_t st, double *row_ss, void *const *events) {
     int rc = experts_check(s);
     if (rc != ODSD_OK) return rc;
     if (s->T == 0) return ODSD_OK;
@@ -698,9 +698,14 @@ int odsd_launch_experts(const odsd_moe_shape *s, const void *x16, const uint64_t
     float *y = (float *)((char *)ws + pl.h_bytes);
     rc = odsd_w4_gate_up_silu(s, x16, table, counts, offsets, slot_token, h16, st);
     if (rc != ODSD_OK) return rc;
+    if (events && hipEventRecord((hipEvent_t)events[0], st) != hipSuccess) return ODSD_ERR_LAUNCH;
     rc = odsd_w4_down(s, h16, table, counts, offsets, y, st);
     if (rc != ODSD_OK) return rc;
-    return launch_combine(s, y, idx, w, perm, table, residual, out_f32, out_act, row_ss, st);
+    if (events && hipEventRecord((hipEvent_t)events[1], st) != hipSuccess) return ODSD_ERR_LAUNCH;
+    rc = launch_combine(s, y, idx, w, perm, table, residual, out_f32, out_act, row_ss, st);
+    if (rc != ODSD_OK) return rc;
+    if (events && hipEventRecord((hipEvent_t)events[2], st) != hipSuccess) return ODSD_ERR_LAUNCH;
+    return ODSD_OK;
 }
 
 extern "C" int odsd_experts_w4(const odsd_moe_shape *s, const void *x_f16, const uint64_t *table,

@@ -29,7 +29,7 @@ def test_version_and_status_strings():
     lib = _lib.load()
     assert lib.odsd_version() == 100
     assert lib.odsd_status_string(0) == b"ok"
-    for code in range(1, 8):
+    for code in range(1, 9):
         assert len(lib.odsd_status_string(code)) > 3
 
 
@@ -74,3 +74,19 @@ def test_argument_checks_need_no_gpu():
     assert lib.odsd_w4_packed_q_bytes(30, 256) == 0
     empty = _lib.MoeShape(0, 256, 8, 2, 256, 1, _lib.DT_BF16, 0)       # T == 0 is a no-op
     assert lib.odsd_dispatch(C.byref(empty), 1 << 20, 1 << 20, 1 << 20, 1 << 20, 1 << 20, 1 << 20, None) == 0
+
+
+def test_static_scratch_call_refuses_what_does_not_fit():
+    """odsd_moe_forward_static returns ODSD_ERR_SCRATCH, before touching the device, for a shape
+    whose workspace is larger than the library's static array."""
+    lib = _lib.load()
+    big = _lib.MoeShape(4096, 4096, 128, 8, 1536, 1, _lib.DT_BF16, 0)
+    assert lib.odsd_moe_workspace_bytes(C.byref(big)) > _lib.STATIC_SCRATCH_BYTES
+    rc = lib.odsd_moe_forward_static(C.byref(big), 1 << 20, None, 1e-6, 1 << 20, 1 << 20, 0, 1 << 20, None,
+                                     None, None, None, None, None, None, None, None)
+    assert rc == 8
+    assert b"scratch" in lib.odsd_status_string(rc)
+    # the header's constant and the binding's agree
+    text = open(os.path.join(ROOT, "include", "odsd_moe.h")).read()
+    m = re.search(r"#define ODSD_STATIC_SCRATCH_BYTES \((\d+)u << (\d+)\)", text)
+    assert m and int(m.group(1)) << int(m.group(2)) == _lib.STATIC_SCRATCH_BYTES
