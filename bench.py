@@ -1,15 +1,22 @@
 #!/usr/bin/env python3
 """Benchmark of the W4 MoE-block hot path on one MI355X.
 
-A step is one whole MoE block (router -> dispatch -> W4 gate_up+SiLU*mul -> W4 down ->
-combine) over one batch of synthetic tokens, through odsd_moe_forward.  The headline
-workload is the Mixtral-8x7B-shaped verify layer with T=160 tokens; `--workload NAME`
-selects another one and `--all` adds the remaining configurations under "workloads".
+A step is one pass of the hot path over one batch of synthetic tokens.  The headline workload is
+the largest single-GPU configuration, the Qwen3-30B-A3B-shaped 48-layer MoE-only stack at T=256
+(15.4 GB of W4 experts resident in HBM; one step = RMSNorm -> router -> dispatch -> W4 gate_up +
+SiLU*mul -> W4 down -> combine -> residual, 48 times); the other four configurations are measured
+the same way and reported under "workloads".  `--workload NAME` measures one configuration only.
 
-The printed JSON line carries, next to the throughput, the roofline of the dominant kernel
-(the gate_up W4 stream for verify shapes: algorithmic bytes / measured kernel time against
-8 TB/s; for the prefill shape algorithmic flops against 2.5 PFLOP/s) and a CPU baseline (the
-oracle's per-expert loop on the host cores over the same inputs).
+Every result carries
+  * the whole-step time (host clock around K back-to-back steps, inputs resident in HBM),
+  * per-kernel GPU times from HIP events: in the timed steps every kernel launch of the library
+    carries its own start / stop events on the launch stream (odsd_moe_forward_events), which the
+    runtime stamps with the kernel's begin and end; nothing is inserted between the kernels, so
+    the kernel times add up to at most the step time,
+  * the roofline of the dominant kernel (verify shapes: the gate_up W4 stream, algorithmic bytes
+    over its event time against 8 TB/s; prefill shape: algorithmic flops against 2.5 PFLOP/s),
+  * a CPU baseline: the oracle's restatement of the reference's per-expert loop on the host cores
+    over the same inputs, with fp32 weights dequantised beforehand.
 """
 import argparse
 import json
@@ -22,111 +29,128 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
-HEADLINE = "mixtral_t160"
-
-# HBM bytes per launch of the gate_up kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
-# runs of this command (summaries and calibration in profiles/w4_gemm_gate_up_hbm_traffic.md):
-# FETCH_SIZE reads half of the bytes a plain 1 GiB device copy moves (factor 2.0), WRITE_SIZE
-# reads them in KiB (factor 1.0).
-MEASURED_TRAFFIC_BYTES = {
-    "mixtral_t160": 260564.9 * 2.0 * 1024 + 8964.6 * 1024,
-}
+HEADLINE = "qwen3_30b_stack48_t256"
+OTHERS = ("mixtral_t160", "mixtral_t5", "qwen3_30b_t64_zipf", "qwen3_235b_t4096")
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
 
 
-def _build_layer(wl, dev, layer=0):
-    import torch
+def _log(msg):
+    print(f"[bench] {msg}", file=sys.stderr, flush=True)
+
+
+def _host_threads():
+    n = os.cpu_count() or 1
+    for var in ("OMP_NUM_THREADS",):
+        try:
+            n = min(n, int(os.environ[var]))
+        except (KeyError, ValueError):
+            pass
+    return max(1, n)
+
+
+def _build_layer(wl, dev, layer=0, keep_canonical=False):
     import on_device_sd_amd as odsd
     from on_device_sd_amd.workloads import LayerInputs
     inp = LayerInputs(wl, dev, layer)
     gate = inp.gate_weight()
     bank = odsd.W4ExpertBank(wl.E, wl.H, wl.I, dev)
+    canon = {}
     for e, gw, uw, dw in inp.experts():
-        bank.load_expert(e, gw, uw, dw)
+        c = bank.load_expert(e, gw, uw, dw, keep_canonical=keep_canonical)
+        if keep_canonical:
+            canon[e] = c
     x = inp.x()
-    return gate, bank, x
+    return gate, bank, x, canon
 
 
-def _clone_bank(bank):
-    return bank.clone()
-
-
-def _event_ms(fn, n):
-    """Average duration of fn() over n launches, each bracketed by its own pair of events on
-    the current stream (the stream the kernels are launched on)."""
+def _dequant_to_host(canon_expert):
+    """fp32 (gate, up, down) weights of one expert on the host.  The arithmetic is the oracle's
+    dequantize_w4, (code - zero) * scale in fp32, done with torch on the device because numpy
+    needs tens of seconds for the larger layers; this is preparation, not part of any timing."""
     import torch
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
-    for i, (a, b) in enumerate(evs):
-        a.record()
-        fn(i)
-        b.record()
-    torch.cuda.synchronize()
-    ts = sorted(a.elapsed_time(b) for a, b in evs)
-    return sum(ts) / len(ts), ts[len(ts) // 2], ts[0]
-
-
-def _event_ms_sequence(stages, n):
-    """Average / median / minimum duration of every stage of a sequence that is launched n times
-    back to back, with an event between consecutive stages (on the launch stream)."""
-    import torch
-    ns = len(stages)
-    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(ns + 1)] for _ in range(n)]
-    for i in range(n):
-        evs[i][0].record()
-        for k, fn in enumerate(stages):
-            fn(i)
-            evs[i][k + 1].record()
-    torch.cuda.synchronize()
     out = []
-    for k in range(ns):
-        ts = sorted(evs[i][k].elapsed_time(evs[i][k + 1]) for i in range(n))
-        out.append((sum(ts) / len(ts), ts[len(ts) // 2], ts[0]))
-    return out
+    for q, s, z in canon_expert:
+        n, kb = q.shape
+        codes = torch.stack((q & 15, q >> 4), dim=-1).view(n, kb * 2).to(torch.float32)
+        g = kb * 2 // 128
+        d = codes.view(n, g, 128) - z.to(torch.float32)[:, :, None]
+        out.append((d * s.to(torch.float32)[:, :, None]).view(n, kb * 2).cpu())
+    return tuple(out)
+
+
+def _stage_stats(per_step):
+    """per_step: list (steps) of lists (stages) of ms -> per-stage average over the steps."""
+    n = len(per_step)
+    return [sum(s[k] for s in per_step) / n for k in range(len(per_step[0]))]
+
+
+def _traffic(wl_name):
+    """HBM bytes per launch of the dominant kernel as measured offline with rocprofv3 --pmc
+    (FETCH_SIZE, WRITE_SIZE) and recorded, with the commit it was measured on, in
+    profiles/hbm_traffic.json; None when there is no record for the workload."""
+    try:
+        rec = json.load(open(TRAFFIC_FILE))[wl_name]
+        return rec["bytes_per_launch"], rec.get("commit")
+    except (OSError, KeyError, ValueError):
+        return None, None
+
+
+def _roofline(wl, kernel_ms, algorithmic_bytes):
+    gu_flops = 4 * wl.pairs * wl.H * wl.I
+    traffic, commit = _traffic(wl.name)
+    if wl.regime == "prefill":
+        ach = gu_flops / (kernel_ms * 1e-3) / 1e12
+        roof = {"bound": "mfma", "kernel": "w4_gemm_prefill_kernel<gate_up>", "achieved": round(ach, 2),
+                "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(ach / MFMA_F16_PEAK_TFLOPS, 4),
+                "traffic": traffic, "algorithmic_flops": gu_flops}
+    else:
+        ach = algorithmic_bytes / (kernel_ms * 1e-3) / 1e9
+        roof = {"bound": "hbm", "kernel": "w4_gemm_kernel<gate_up>", "achieved": round(ach, 1),
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4),
+                "traffic": traffic, "algorithmic_bytes": int(algorithmic_bytes)}
+    if commit:
+        roof["traffic_measured_at_commit"] = commit
+    roof["kernel_ms"] = round(kernel_ms, 5)
+    return roof
 
 
 def bench_layer(wl, dev, steps, warmup, with_cpu):
+    """One MoE layer; weight replicas are rotated from step to step so that the 256 MB memory-side
+    cache cannot hold the weight stream."""
     import torch
-    from on_device_sd_amd import ops
-    gate, bank, x = _build_layer(wl, dev)
-    # rotate over weight replicas so that the 256 MB memory-side cache cannot hold the stream
+    from on_device_sd_amd import _hip, _lib, ops
+    _log(f"{wl.name}: building the layer")
+    gate, bank, x, canon = _build_layer(wl, dev, keep_canonical=with_cpu)
     layer_bytes = wl.E * wl.expert_w4_bytes
     n_rep = max(2, min(4, -(-(1 << 30) // layer_bytes)))
-    banks = [bank] + [_clone_bank(bank) for _ in range(n_rep - 1)]
+    banks = [bank] + [bank.clone() for _ in range(n_rep - 1)]
     tables = [b.table() for b in banks]
     plan = ops.MoeForwardPlan(wl.T, wl.H, wl.E, wl.K, wl.I, wl.renorm, wl.act_dtype, dev)
-
-    def step(i):
-        plan.run(x, gate, tables[i % n_rep])
-
+    # timed region: K whole-block calls back to back
     for i in range(warmup):
-        step(i)
+        plan.run(x, gate, tables[i % n_rep])
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(steps):
-        step(i)
+        plan.run(x, gate, tables[i % n_rep])
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) * 1e3 / steps
+
+    # the same K steps once more with every kernel launch carrying its start / stop events (the
+    # runtime's handling of those events makes the step itself slower, the kernels are not)
+    events = [_hip.EventList(2 * _lib.N_KERNELS) for _ in range(steps)]
+    masks = [0] * steps
+    plan.run_events(events[0], x, gate, tables[0])
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        masks[i] = plan.run_events(events[i], x, gate, tables[i % n_rep])
+    torch.cuda.synchronize()
+    ms_events = (time.perf_counter() - t0) * 1e3 / steps
+    stage_ms = _stage_stats([ev.kernel_ms(m) for ev, m in zip(events, masks)])
     counts = plan.counts.cpu()
     active = int((counts > 0).sum())
 
-    # per-kernel durations through the stage entry points
-    idx, w, _, x16 = ops.router_topk(x, gate, wl.K, wl.renorm, want_f16=True)
-    disp = ops.dispatch(idx, wl.E)
-    st = ops.ExpertStages(wl.T, wl.H, wl.E, wl.K, wl.I, wl.act_dtype, dev)
-    out32 = torch.empty(wl.T, wl.H, dtype=torch.float32, device=dev)
-    n = max(steps, 10)
-    for i in range(3):
-        st.gate_up(x16, tables[i % n_rep], disp); st.down(tables[i % n_rep], disp)
-    # every stage bracketed by its own events INSIDE the sequence of a whole step (router ->
-    # dispatch -> gate_up -> down -> combine), so that each kernel is timed under the clocks and
-    # cache state it sees in the timed region, not in a loop of its own
-    stages = [
-        lambda i: ops.router_topk(x, gate, wl.K, wl.renorm, want_f16=True),
-        lambda i: ops.dispatch(idx, wl.E),
-        lambda i: st.gate_up(x16, tables[i % n_rep], disp),
-        lambda i: st.down(tables[i % n_rep], disp),
-        lambda i: st.combine(idx, w, disp, tables[0], out_f32=out32),
-    ]
-    k_rt, k_dp, k_gu, k_dn, k_cb = _event_ms_sequence(stages, n)
     # the two-call path of the reference engine loops: route_experts, the host reads the
     # activated set, forward_moe (reported beside the whole-block call, never as `value`)
     import on_device_sd_amd as odsd
@@ -147,58 +171,51 @@ def bench_layer(wl, dev, steps, warmup, with_cpu):
         engine_step(i)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for i in range(n):
+    for i in range(steps):
         engine_step(i)
     torch.cuda.synchronize()
-    engine_ms = (time.perf_counter() - t0) * 1e3 / n
+    engine_ms = (time.perf_counter() - t0) * 1e3 / steps
 
+    k = dict(zip(_lib.KERNEL_NAMES, stage_ms))
     gu_bytes = active * (wl.expert_w4_bytes * 2 // 3)
-    gu_flops = 4 * wl.pairs * wl.H * wl.I
-    if wl.regime == "prefill":
-        ach = gu_flops / (k_gu[0] * 1e-3) / 1e12
-        roof = {"bound": "mfma", "kernel": "w4_gemm_kernel<gate_up>", "achieved": round(ach, 2),
-                "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(ach / MFMA_F16_PEAK_TFLOPS, 4),
-                "traffic": None}
-    else:
-        ach = gu_bytes / (k_gu[0] * 1e-3) / 1e9
-        roof = {"bound": "hbm", "kernel": "w4_gemm_kernel<gate_up>", "achieved": round(ach, 1),
-                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4),
-                "traffic": MEASURED_TRAFFIC_BYTES.get(wl.name)}
-        roof["algorithmic_bytes"] = gu_bytes
-    roof["kernel_ms"] = round(k_gu[0], 4)
-    layer_bytes_alg = wl.algorithmic_bytes(active)
     res = {
         "workload": wl.name, "T": wl.T, "H": wl.H, "E": wl.E, "K": wl.K, "I": wl.I,
-        "tokens_per_s": wl.T / (ms * 1e-3), "ms_per_step": ms, "engine_path_ms": engine_ms,
-        "active_experts": active,
-        "max_rows_per_expert": int(counts.max()), "weight_replicas": n_rep,
-        "layer_hbm_frac": layer_bytes_alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-        "layer_mfma_frac": wl.algorithmic_flops() / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS,
-        "kernel_ms": {"router": k_rt[0], "dispatch": k_dp[0], "gate_up": k_gu[0], "down": k_dn[0],
-                      "combine": k_cb[0]},
-        "roofline": roof,
+        "tokens_per_s": round(wl.T / (ms * 1e-3), 1), "ms_per_step": round(ms, 5),
+        "ms_per_step_with_kernel_events": round(ms_events, 5), "engine_path_ms": round(engine_ms, 5),
+        "active_experts": active, "max_rows_per_expert": int(counts.max()), "weight_replicas": n_rep,
+        "layer_hbm_frac": round(wl.algorithmic_bytes(active) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+        "layer_mfma_frac": round(wl.algorithmic_flops() / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
+        "kernel_ms": {n: round(v, 5) for n, v in k.items()},
+        "kernel_ms_sum": round(sum(stage_ms), 5),
+        "roofline": _roofline(wl, k["gate_up"], gu_bytes),
     }
+    del runner, placements, plan, banks, tables
     if with_cpu:
-        res["cpu_baseline"] = cpu_baseline(wl, gate, bank, x)
+        res["cpu_baseline"] = cpu_baseline_layer(wl, gate, x, canon)
     return res
 
 
-def bench_stack(wl, dev, steps, warmup):
+def bench_stack(wl, dev, steps, warmup, with_cpu, cpu_layers=4):
     """48-layer RMSNorm -> MoE -> residual stack, all experts resident."""
     import torch
     import on_device_sd_amd as odsd
-    from on_device_sd_amd.workloads import LayerInputs
+    from on_device_sd_amd import _hip, _lib
     cfg = odsd.MoEConfig(hidden_size=wl.H, num_hidden_layers=wl.layers, num_experts=wl.E,
                          num_experts_per_token=wl.K, moe_intermediate_size=wl.I,
                          norm_topk_prob=wl.renorm)
-    gates, banks, x = [], [], None
+    _log(f"{wl.name}: building {wl.layers} layers")
+    gates, banks, x, canon_layers = [], [], None, []
     for l in range(wl.layers):
-        g, b, xl = _build_layer(wl, dev, l)
+        keep = with_cpu and l < cpu_layers
+        g, b, xl, canon = _build_layer(wl, dev, l, keep_canonical=keep)
         gates.append(g); banks.append(b)
+        if keep:
+            canon_layers.append(canon)
         if l == 0:
             x = xl
     norms = [torch.ones(wl.H, dtype=wl.act_dtype, device=dev) for _ in range(wl.layers)]
     stack = odsd.MoEOnlyStack(cfg, gates, norms, banks, wl.T)
+    # timed region: K passes through the stack, as eager launches and as one HIP graph
     out = {}
     for mode in ("eager", "graph"):
         if mode == "graph":
@@ -212,61 +229,147 @@ def bench_stack(wl, dev, steps, warmup):
         torch.cuda.synchronize()
         out[mode] = (time.perf_counter() - t0) * 1e3 / steps
     ms = min(out.values())
-    total_bytes = wl.layers * wl.algorithmic_bytes(wl.E, out_bytes=2)
-    return {"workload": wl.name, "T": wl.T, "layers": wl.layers, "ms_per_step": ms,
-            "ms_eager": out["eager"], "ms_graph": out["graph"], "tokens_per_s": wl.T / (ms * 1e-3),
-            "resident_weight_gb": wl.layers * wl.E * wl.expert_w4_bytes / 1e9,
-            "layer_hbm_frac": total_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    stack.graph = None
+
+    # the same K steps once more (eager) with every kernel launch carrying its start / stop events
+    events = [[_hip.EventList(2 * _lib.N_KERNELS) for _ in range(wl.layers)] for _ in range(steps)]
+    masks = [None] * steps
+    stack.forward_events(x, events[0])
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        masks[i] = stack.forward_events(x, events[i])
+    torch.cuda.synchronize()
+    ms_events = (time.perf_counter() - t0) * 1e3 / steps
+    # per layer: the kernel times; per step: their sums over the layers
+    per_step = []
+    for i in range(steps):
+        tot = [0.0] * _lib.N_KERNELS
+        for l in range(wl.layers):
+            for s, v in enumerate(events[i][l].kernel_ms(masks[i][l])):
+                tot[s] += v
+        per_step.append(tot)
+    stage_ms = _stage_stats(per_step)
+
+    k = dict(zip(_lib.KERNEL_NAMES, stage_ms))
+    # active experts per layer: re-run the layers' routing through the whole-block outputs
+    active = _stack_active_experts(stack, x, wl)
+    gu_bytes_total = sum(active) * (wl.expert_w4_bytes * 2 // 3)
+    alg_bytes = sum(wl.algorithmic_bytes(a, out_bytes=2) for a in active)
+    res = {
+        "workload": wl.name, "T": wl.T, "H": wl.H, "E": wl.E, "K": wl.K, "I": wl.I, "layers": wl.layers,
+        "tokens_per_s": round(wl.T / (ms * 1e-3), 1), "ms_per_step": round(ms, 5),
+        "ms_per_step_eager": round(out["eager"], 5), "ms_per_step_graph": round(out["graph"], 5),
+        "ms_per_step_with_kernel_events": round(ms_events, 5),
+        "resident_weight_gb": round(wl.layers * wl.E * wl.expert_w4_bytes / 1e9, 3),
+        "active_experts_per_layer_mean": round(sum(active) / len(active), 2),
+        "layer_hbm_frac": round(alg_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+        "kernel_ms": {n: round(v, 5) for n, v in k.items()},
+        "kernel_ms_sum": round(sum(stage_ms), 5),
+        "kernel_ms_note": "sums over the 48 layers of one step",
+        # the dominant kernel runs once per layer: average launch = sum over layers / layers
+        "roofline": _roofline(wl, k["gate_up"] / wl.layers, gu_bytes_total / wl.layers),
+    }
+    del stack, events
+    if with_cpu:
+        res["cpu_baseline"] = cpu_baseline_stack(wl, gates, norms, x, canon_layers)
+    return res
 
 
-def cpu_baseline(wl, gate, bank, x):
-    """The reference's CPU MoE path restated by the oracle (router F.linear -> top-k ->
-    per-expert expert_forward loop -> weighted accumulate) on the host cores, fp32, with the
-    W4 weights dequantised once beforehand.  Bounded: only as many experts are dequantised
-    and timed as fit a ~20 s budget; the rate is scaled by pairs processed."""
+def _stack_active_experts(stack, x, wl):
+    """Experts with at least one token, per layer, from the counts the whole-block call returns."""
+    import torch
+    from on_device_sd_amd import ops
+    plan = ops.MoeForwardPlan(wl.T, wl.H, wl.E, wl.K, wl.I, wl.renorm, wl.act_dtype, x.device,
+                              want_f32=False, want_act=True)
+    h = x.clone()
+    active = []
+    for l in range(stack.L):
+        o = plan.run(h, stack.gate[l], stack.tables[l], stack.norm[l], stack.config.rms_norm_eps,
+                     add_residual=True)
+        active.append(int((o.counts > 0).sum()))
+        h = o.out_act.clone()
+    torch.cuda.synchronize()
+    return active
+
+
+def _time_cpu(run, budget_s, min_runs=2, max_runs=10):
+    run()                                         # warm-up (thread pool, page faults)
+    ts = []
+    t_end = time.perf_counter() + budget_s
+    while len(ts) < min_runs or (len(ts) < max_runs and time.perf_counter() < t_end):
+        t0 = time.perf_counter(); run(); ts.append(time.perf_counter() - t0)
+    return sorted(ts)[len(ts) // 2], len(ts)
+
+
+def cpu_baseline_layer(wl, gate, x, canon):
+    """The reference's CPU MoE path restated by the oracle (router F.linear -> top-k -> per-expert
+    expert_forward loop -> weighted accumulate) on the host cores, fp32, over the whole layer:
+    every active expert, weights dequantised once beforehand."""
     import numpy as np
     import torch
     from oracle import moe_oracle as orc
-    from tests.helpers import unpack_bank_expert
-    cores = os.cpu_count() or 1
+    cores = _host_threads()
     torch.set_num_threads(cores)
     xc, gc = x.cpu(), gate.cpu()
     idx, w = orc.route(orc.router_logits(xc, gc), wl.K, wl.renorm)
-    counts = np.bincount(idx.reshape(-1), minlength=wl.E)
-    order = [int(e) for e in np.argsort(-counts) if counts[e] > 0]
-    budget_weights = 4.0e8          # dequantised fp32 weights held at once (1.6 GB)
-    per_expert = 3 * wl.H * wl.I
-    n_exp = max(1, min(len(order), int(budget_weights // per_expert)))
-    chosen = order[:n_exp]
-    experts = {e: unpack_bank_expert(bank, e).dequant() for e in chosen}
-    pairs = int(sum(counts[e] for e in chosen))
+    active = [int(e) for e in np.unique(idx)]
+    _log(f"{wl.name}: CPU baseline, dequantising {len(active)} experts")
+    experts = {e: _dequant_to_host(canon[e]) for e in active}
+    canon.clear()
 
     def run():
-        return orc.moe_forward(xc, idx, w, experts)
-    for _ in range(2):
-        run()
-    ts = []
-    t_end = time.perf_counter() + 15.0
-    while len(ts) < 5 or (len(ts) < 20 and time.perf_counter() < t_end and sum(ts) < 5.0):
-        t0 = time.perf_counter(); run(); ts.append(time.perf_counter() - t0)
-        if time.perf_counter() > t_end:
-            break
-    med = sorted(ts)[len(ts) // 2]
-    # time for the whole layer = time for the sampled pairs scaled to all pairs
-    layer_s = med * (wl.pairs / max(pairs, 1))
-    return {"value": wl.T / layer_s, "unit": "tokens/s", "cores": cores, "kind": "port",
-            "sample": f"{n_exp} of {len(order)} active experts ({pairs} of {wl.pairs} token-expert pairs), "
-                      f"fp32 dequantised weights, median of {len(ts)} runs, scaled by pairs"}
+        i2, w2 = orc.route(orc.router_logits(xc, gc), wl.K, wl.renorm)
+        return orc.moe_forward(xc, i2, w2, experts)
+    med, n = _time_cpu(run, budget_s=12.0)
+    return {"value": round(wl.T / med, 2), "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"the whole layer: all {len(active)} active experts, {wl.pairs} token-expert pairs, "
+                      f"fp32 dequantised weights in host memory, median of {n} runs"}
+
+
+def cpu_baseline_stack(wl, gates, norms, x, canon_layers):
+    """The first n layers of the stack on the host cores (RMSNorm -> router -> per-expert loop ->
+    combine -> residual per layer), scaled by layers/n."""
+    import torch
+    from oracle import moe_oracle as orc
+    cores = _host_threads()
+    torch.set_num_threads(cores)
+    n = len(canon_layers)
+    _log(f"{wl.name}: CPU baseline, dequantising {n} layers")
+    layers = []
+    for l in range(n):
+        experts = {e: _dequant_to_host(c) for e, c in canon_layers[l].items()}
+        canon_layers[l].clear()
+        layers.append((norms[l].cpu(), gates[l].cpu(), experts))
+    xc = x.cpu()
+
+    def run():
+        h = xc
+        for nw, gw, experts in layers:
+            h = orc.moe_only_layer(h, nw, gw, experts, wl.K, wl.renorm)[0]
+        return h
+    med, runs = _time_cpu(run, budget_s=12.0)
+    stack_s = med * wl.layers / n
+    return {"value": round(wl.T / stack_s, 2), "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"layers 0..{n - 1} of {wl.layers} (all 128 experts each, fp32 dequantised weights in "
+                      f"host memory), median of {runs} runs, time scaled by {wl.layers}/{n}"}
+
+
+def run_workload(wl, dev, steps, warmup, with_cpu):
+    import torch
+    res = bench_stack(wl, dev, steps, warmup, with_cpu) if wl.layers > 1 else \
+        bench_layer(wl, dev, steps, warmup, with_cpu)
+    torch.cuda.empty_cache()
+    return res
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default=HEADLINE)
-    ap.add_argument("--all", action="store_true", help="also run the other configurations")
-    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default=None, help="measure this configuration only")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (use --gpus 1)", file=sys.stderr)
@@ -279,34 +382,24 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
-    wl = CONFIGS[args.workload]
-    if wl.layers > 1:
-        main_res = bench_stack(wl, dev, max(3, args.steps // 10), max(1, args.warmup // 5))
-    else:
-        main_res = bench_layer(wl, dev, args.steps, args.warmup, not args.no_cpu)
+    head = CONFIGS[args.workload or HEADLINE]
+    main_res = run_workload(head, dev, args.steps, args.warmup, not args.no_cpu)
     line = {
-        "metric": "int4 MoE-layer tokens/s", "value": round(main_res["tokens_per_s"], 1), "unit": "tokens/s",
+        "metric": "int4 MoE-layer tokens/s", "value": main_res["tokens_per_s"], "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(main_res["ms_per_step"], 5), "higher_is_better": True, "scaling": "weak",
+        "ms_per_step": main_res["ms_per_step"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f16 MFMA / fp32 accumulate on int4 weights (bf16 activations in and out)",
         "data": "synthetic",
-        "config": {"workload": wl.name, "T": wl.T, "hidden": wl.H, "experts": wl.E, "top_k": wl.K,
-                   "intermediate": wl.I, "renorm": wl.renorm, "weights": "W4 group-128 asymmetric fp16 scale/zero"},
+        "config": {"workload": head.name, "T": head.T, "hidden": head.H, "experts": head.E, "top_k": head.K,
+                   "intermediate": head.I, "layers": head.layers, "renorm": head.renorm,
+                   "weights": "W4 group-128 asymmetric fp16 scale/zero"},
         "roofline": main_res.get("roofline"),
         "cpu_baseline": main_res.get("cpu_baseline"),
         "detail": {k: v for k, v in main_res.items() if k not in ("roofline", "cpu_baseline")},
     }
-    if args.all:
-        others = []
-        for name, w2 in CONFIGS.items():
-            if name == wl.name or name == "tiny":
-                continue
-            torch.cuda.empty_cache()
-            if w2.layers > 1:
-                others.append(bench_stack(w2, dev, 5, 2))
-            else:
-                others.append(bench_layer(w2, dev, max(10, args.steps // 2), args.warmup, False))
-        line["workloads"] = others
+    if args.workload is None:
+        line["workloads"] = [run_workload(CONFIGS[name], dev, args.steps, args.warmup, not args.no_cpu)
+                             for name in OTHERS]
     print(json.dumps(line))
 
 

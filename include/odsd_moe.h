@@ -199,6 +199,30 @@ int odsd_moe_forward(const odsd_moe_shape *s, const void *x, const void *norm_we
                      const double *row_sumsq_in, double *row_sumsq_out,
                      void *workspace, size_t workspace_bytes, void *stream);
 
+/* The same call with every kernel timed, for measurement (no counterpart in the reference):
+ * events = 2 * ODSD_N_KERNELS hipEvent_t handles created by the caller; the launch of kernel slot k
+ * carries events[2k] and events[2k+1] as its start and stop events (hipExtLaunchKernel), so after
+ * the stream has been synchronised hipEventElapsedTime(events[2k], events[2k+1]) is that kernel's
+ * own duration; nothing is inserted between the kernels.  *launched_mask gets bit k set for every
+ * slot that was launched (a block without a stand-alone RMSNorm leaves slot 0 out); the events of
+ * the other slots are not touched.  Results are those of odsd_moe_forward. */
+enum {
+    ODSD_KERNEL_NORM = 0,           /* stand-alone RMSNorm                          */
+    ODSD_KERNEL_ROUTER_LOGITS = 1,  /* fp64 logit partials (+ fp16 copy of x)       */
+    ODSD_KERNEL_ROUTER_TOPK = 2,
+    ODSD_KERNEL_DISPATCH = 3,
+    ODSD_KERNEL_GATE_UP = 4,
+    ODSD_KERNEL_DOWN = 5,
+    ODSD_KERNEL_COMBINE = 6,
+    ODSD_N_KERNELS = 7
+};
+int odsd_moe_forward_events(const odsd_moe_shape *s, const void *x, const void *norm_weight,
+                            float eps, const void *gate_w, const uint64_t *table,
+                            int32_t add_residual, float *out_f32, void *out_act,
+                            const double *row_sumsq_in, double *row_sumsq_out,
+                            void *workspace, size_t workspace_bytes, void *stream,
+                            void *const *events, uint32_t *launched_mask);
+
 /* odsd_moe_forward without a workspace argument and without any allocation, for callers that
  * cannot call hipMalloc: code under HIP graph capture, tight serving loops, harnesses that
  * forbid it.  It has no counterpart in the reference.  The workspace is a device array inside

@@ -53,10 +53,14 @@ SIGNATURES = {
     "odsd_moe_workspace_bytes": (C.c_size_t, [_SP]),
     "odsd_moe_forward": (C.c_int, [_SP, _P, _P, C.c_float, _P, _P, C.c_int32, _P, _P, _P, _P, _P, _P,
                                    _P, _P, _P, _P, C.c_size_t, _P]),
+    "odsd_moe_forward_events": (C.c_int, [_SP, _P, _P, C.c_float, _P, _P, C.c_int32, _P, _P, _P, _P, _P,
+                                          C.c_size_t, _P, _P, _P]),
     "odsd_moe_forward_static": (C.c_int, [_SP, _P, _P, C.c_float, _P, _P, C.c_int32, _P, _P, _P, _P, _P,
                                           _P, _P, _P, _P, _P]),
 }
 
+N_KERNELS = 7                          # ODSD_N_KERNELS
+KERNEL_NAMES = ("norm", "router_logits", "router_topk", "dispatch", "gate_up", "down", "combine")
 STATIC_SCRATCH_BYTES = 64 << 20        # ODSD_STATIC_SCRATCH_BYTES
 
 _lib: Optional[C.CDLL] = None

@@ -56,14 +56,15 @@ extern "C" size_t odsd_moe_workspace_bytes(const odsd_moe_shape *s) {
     return moe_layout(s).total;
 }
 
-// One whole block.  `events` (optional, ODSD_N_STAGES + 1 hipEvent_t handles): event 0 is recorded
-// before the first launch and event k + 1 after the launches of stage k .
+thread_local OdsdProf *odsd_prof = nullptr;
+
+// One whole block.
 static int moe_forward_impl(const odsd_moe_shape *s, const void *x, const void *norm_weight, float eps,
                             const void *gate_w, const uint64_t *table, int32_t add_residual,
                             float *out_f32, void *out_act, int32_t *out_idx, float *out_w,
                             int32_t *out_counts, int32_t *out_offsets, int32_t *out_perm,
                             const double *row_sumsq_in, double *row_sumsq_out,
-                            void *workspace, size_t workspace_bytes, void *stream, void *const *events) {
+                            void *workspace, size_t workspace_bytes, void *stream) {
     if (!s) return ODSD_ERR_NULL;
     const size_t need = odsd_moe_workspace_bytes(s);
     if (need == 0) return ODSD_ERR_SHAPE;
@@ -82,12 +83,6 @@ static int moe_forward_impl(const odsd_moe_shape *s, const void *x, const void *
     int32_t *inv = (int32_t *)(ws + l.inv);
     int32_t *slot_token = (int32_t *)(ws + l.slot_token);
     void *x16 = ws + l.x16;
-    int n_ev = 0;
-#define ODSD_STAGE_DONE()                                                                        \
-    do {                                                                                         \
-        if (events && hipEventRecord((hipEvent_t)events[n_ev++], st) != hipSuccess) return ODSD_ERR_LAUNCH; \
-    } while (0)
-    ODSD_STAGE_DONE();
 
     // RMSNorm: with the row statistics at hand (left by the previous block's combine) the router
     // kernel normalises on the fly; otherwise the stand-alone kernel runs first
@@ -99,19 +94,15 @@ static int moe_forward_impl(const odsd_moe_shape *s, const void *x, const void *
         if (rc != ODSD_OK) return rc;
         xin = ws + l.xn;
     }
-    ODSD_STAGE_DONE();   // ODSD_STAGE_NORM
     int rc = odsd_launch_router(s, xin, gate_w, idx, w, nullptr, x16, ws + l.router,
                                 l.xn - l.router, st, fold ? row_sumsq_in : nullptr, norm_weight, eps,
                                 nullptr, nullptr);
     if (rc != ODSD_OK) return rc;
-    ODSD_STAGE_DONE();   // ODSD_STAGE_ROUTER
     rc = odsd_launch_dispatch(s, idx, counts, offsets, perm, inv, slot_token, st);
     if (rc != ODSD_OK) return rc;
-    ODSD_STAGE_DONE();   // ODSD_STAGE_DISPATCH
     return odsd_launch_experts(s, x16, table, idx, w, counts, offsets, perm, slot_token,
                                add_residual ? x : nullptr, out_f32, out_act, ws + l.experts,
-                               l.total - l.experts, st, row_sumsq_out, events ? events + n_ev : nullptr);
-#undef ODSD_STAGE_DONE
+                               l.total - l.experts, st, row_sumsq_out);
 }
 
 extern "C" int odsd_moe_forward(const odsd_moe_shape *s, const void *x, const void *norm_weight, float eps,
@@ -122,7 +113,26 @@ extern "C" int odsd_moe_forward(const odsd_moe_shape *s, const void *x, const vo
                                 void *workspace, size_t workspace_bytes, void *stream) {
     return moe_forward_impl(s, x, norm_weight, eps, gate_w, table, add_residual, out_f32, out_act, out_idx,
                             out_w, out_counts, out_offsets, out_perm, row_sumsq_in, row_sumsq_out,
-                            workspace, workspace_bytes, stream, nullptr);
+                            workspace, workspace_bytes, stream);
+}
+
+extern "C" int odsd_moe_forward_events(const odsd_moe_shape *s, const void *x, const void *norm_weight,
+                                       float eps, const void *gate_w, const uint64_t *table,
+                                       int32_t add_residual, float *out_f32, void *out_act,
+                                       const double *row_sumsq_in, double *row_sumsq_out,
+                                       void *workspace, size_t workspace_bytes, void *stream,
+                                       void *const *events, uint32_t *launched_mask) {
+    if (!events || !launched_mask) return ODSD_ERR_NULL;
+    for (int i = 0; i < 2 * ODSD_N_KERNELS; ++i)
+        if (!events[i]) return ODSD_ERR_NULL;
+    OdsdProf prof{events, 0u};
+    odsd_prof = &prof;
+    const int rc = moe_forward_impl(s, x, norm_weight, eps, gate_w, table, add_residual, out_f32, out_act,
+                                    nullptr, nullptr, nullptr, nullptr, nullptr, row_sumsq_in, row_sumsq_out,
+                                    workspace, workspace_bytes, stream);
+    odsd_prof = nullptr;
+    *launched_mask = prof.launched;
+    return rc;
 }
 
 // ---- the whole block for callers that cannot allocate -------------------------------------------
@@ -170,5 +180,5 @@ extern "C" int odsd_moe_forward_static(const odsd_moe_shape *s, const void *x, c
     // zero and the previous call's contents are simply overwritten
     return moe_forward_impl(s, x, norm_weight, eps, gate_w, table, add_residual, out_f32, out_act, out_idx,
                             out_w, out_counts, out_offsets, out_perm, row_sumsq_in, row_sumsq_out, ws,
-                            (size_t)ODSD_STATIC_SCRATCH_BYTES, stream, nullptr);
+                            (size_t)ODSD_STATIC_SCRATCH_BYTES, stream);
 }

@@ -1,6 +1,7 @@
 // Shared device helpers for the gfx950 MoE kernels (64-wide wavefronts throughout).
 #pragma once
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 
 #include "../../include/odsd_moe.h"
@@ -80,6 +81,34 @@ __device__ __forceinline__ int mask_rank(uint64_t mask) {
 }
 
 // ---- host-side launch plumbing shared by the entry points ----------------------------------
+// Kernel timing for odsd_moe_forward_events: while a call of that entry point is running on a host
+// thread, `odsd_prof` points at its context and every kernel launch of the library on that thread
+// passes the start / stop events of its kernel slot to the runtime, which stamps them with the
+// kernel's own begin and end times (no marker packets between the kernels).
+struct OdsdProf {
+    void *const *events;    // [2 * ODSD_N_KERNELS]: start, stop per kernel slot
+    uint32_t launched;      // bit k: slot k was launched
+};
+extern thread_local OdsdProf *odsd_prof;
+static inline void odsd_prof_events(int slot, hipEvent_t *start, hipEvent_t *stop) {
+    if (odsd_prof) {
+        *start = (hipEvent_t)odsd_prof->events[2 * slot];
+        *stop = (hipEvent_t)odsd_prof->events[2 * slot + 1];
+        odsd_prof->launched |= 1u << slot;
+    }
+}
+// KERNEL goes in parentheses when its template arguments contain commas
+#define ODSD_LAUNCH(SLOT, KERNEL, GRID, BLOCK, STREAM, ...)                                         \
+    do {                                                                                            \
+        if (odsd_prof) {                                                                            \
+            hipEvent_t ev0_ = nullptr, ev1_ = nullptr;                                              \
+            odsd_prof_events(SLOT, &ev0_, &ev1_);                                                   \
+            hipExtLaunchKernelGGL(KERNEL, dim3(GRID), dim3(BLOCK), 0, STREAM, ev0_, ev1_, 0, __VA_ARGS__); \
+        } else {                                                                                    \
+            hipLaunchKernelGGL(KERNEL, dim3(GRID), dim3(BLOCK), 0, STREAM, __VA_ARGS__);            \
+        }                                                                                           \
+    } while (0)
+
 #define ODSD_CHECK_LAUNCH()                                   \
     do {                                                      \
         if (hipGetLastError() != hipSuccess) return ODSD_ERR_LAUNCH; \
@@ -107,5 +136,4 @@ int odsd_launch_experts(const odsd_moe_shape *s, const void *x16, const uint64_t
                         const int32_t *idx, const float *w, const int32_t *counts,
                         const int32_t *offsets, const int32_t *perm, const int32_t *slot_token,
                         const void *residual, float *out_f32, void *out_act, void *ws,
-                        size_t ws_bytes, hipStream_t st, double *row_ss,
-                        void *const *events = nullptr);   // 3 events: after gate_up, down, combine
+                        size_t ws_bytes, hipStream_t st, double *row_ss);

@@ -107,8 +107,9 @@ int odsd_launch_dispatch(const odsd_moe_shape *s, const int32_t *idx, int32_t *c
     const int threads = P <= 4096 ? 256 : 1024;
     const int nwaves = threads / 64;
     const int iters = (((P + nwaves - 1) / nwaves + 63) & ~63) / 64;   // 64-pair chunks per wavefront
-#define DISPATCH_GO(IT) \
-    dispatch_kernel<IT><<<s->E, threads, 0, st>>>(idx, P, s->K, s->E, counts, offsets, perm, inv, slot_token)
+#define DISPATCH_GO(IT)                                                                            \
+    ODSD_LAUNCH(ODSD_KERNEL_DISPATCH, dispatch_kernel<IT>, s->E, threads, st, idx, P, s->K, s->E, counts, \
+                offsets, perm, inv, slot_token)
     if (iters <= 2) DISPATCH_GO(2);
     else if (iters <= 8) DISPATCH_GO(8);
     else if (iters <= 32) DISPATCH_GO(32);

@@ -22,8 +22,6 @@
 // and the indexed "+=" combine (:363, :376).
 #include "w4_gemm.h"
 
-#include <stdlib.h>
-
 // NB    16-row weight blocks per wavefront          MB  16-row token blocks per pass
 // DEPTH groups of weight loads kept in flight       NA  blocks expanded to fp16 at a time
 // WK    wavefronts of a workgroup that split the reduction dimension among themselves
@@ -164,6 +162,17 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
                 if (DIRECT) {
                     wq[buf][i] = __builtin_nontemporal_load((const global_u4 *)(qp_c + (wq_off[i] + gc * 1024u)));
                     wsz[buf][i] = *(const global_u32 *)(szp_c + (sz_off[i] + gc * 64u));
+                } else if (MODE == 1) {
+                    // The ring refills past the last group are still issued (the loop body is
+                    // branch-free).  The down projection's reductions are short (6 groups at I = 768,
+                    // so 2 refills in 8 loads would be wasted): there they go to an offset outside
+                    // the buffer, which returns zeros without touching memory (the range check of a
+                    // raw buffer looks at the per-lane offset only), where a clamped address reads
+                    // the last tile again.  At the cost of a select per load; with the long
+                    // reductions of gate_up the select costs more than the few tiles it saves.
+                    const bool live = g < g_end;
+                    wq[buf][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_q, (int)(live ? wq_off[i] : 0xFFFFFFF0u), (int)(gc * 1024u), 2 /* nt */);
+                    wsz[buf][i] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_sz, (int)(live ? sz_off[i] : 0xFFFFFFF0u), (int)(gc * 64u), 0);
                 } else {
                     wq[buf][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_q, (int)wq_off[i], (int)(gc * 1024u), 2 /* nt */);
                     wsz[buf][i] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_sz, (int)sz_off[i], (int)(gc * 64u), 0);
@@ -186,7 +195,7 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
             for (int i = 0; i < XPT; ++i) {
                 // piece i covers ROWS_PER_PIECE rows from row ROWS_PER_PIECE * i on: nothing to
                 // fetch for a token block without rows
-                if (i * ROWS_PER_PIECE < mcnt_s) {
+                if (i * ROWS_PER_PIECE < mcnt_s && (MODE == 0 || g < g_end)) {
                     lds_void *dst = (lds_void *)(xs_raw + buf * (16 * MB * 256) + (i * 64 * WAVES + wave * 64) * 16);
                     dma16_to_lds(xg, st_off[i], dst);
                 }
@@ -452,7 +461,6 @@ struct ExpertsPlan {
     int KS;          // split of the down projection's reduction dimension across workgroups
     int PS_gu, PS_dn;  // prefill tile kernel: workgroups sharing the row passes of one tile
     int tile;        // MB == 8: the 256 x 256 tile kernel instead of the streaming kernel
-    int stream_nb4;  // MB == 8 streaming: 4 weight blocks per wavefront (comparison runs only)
     int y_f16;       // down-projection outputs kept as fp16 (prefill tile kernel) instead of fp32 partials
     size_t h_bytes, y_bytes;
 };
@@ -460,8 +468,6 @@ struct ExpertsPlan {
 // Choices are functions of the shape only (the per-expert counts live on the device).
 static ExpertsPlan experts_plan(const odsd_moe_shape *s) {
     ExpertsPlan p;
-    // tuning overrides for experiments: ODSD_GEMM_NB (2 or 4), ODSD_GEMM_KS (down-projection splits)
-    static const int env_nb = getenv("ODSD_GEMM_NB") ? atoi(getenv("ODSD_GEMM_NB")) : 0;
     const long P = (long)s->T * s->K;
     const long mean_rows = (P + s->E - 1) / s->E;
     // token blocks per pass follow the mean number of rows per expert; an expert with more
@@ -473,13 +479,6 @@ static ExpertsPlan experts_plan(const odsd_moe_shape *s) {
     else if (s->T <= 32 || mean_rows <= 16) p.MB = 2;
     else if (mean_rows <= 52) p.MB = 4;
     else { p.MB = 8; p.tile = mean_rows > 136; }
-    // tuning overrides for experiments: ODSD_GEMM_MB (1, 2, 4, 8), ODSD_GEMM_PREFILL (with 8 token
-    // blocks: 1 tile kernel, 2 streaming kernel, 0 streaming kernel with 4 weight blocks per wavefront)
-    static const int env_mb = getenv("ODSD_GEMM_MB") ? atoi(getenv("ODSD_GEMM_MB")) : 0;
-    if (env_mb == 1 || env_mb == 2 || env_mb == 4 || env_mb == 8) { p.MB = env_mb; p.tile = env_mb == 8 && mean_rows > 136; }
-    static const int env_pf = getenv("ODSD_GEMM_PREFILL") ? atoi(getenv("ODSD_GEMM_PREFILL")) : -1;
-    p.stream_nb4 = 0;
-    if (p.MB == 8 && env_pf >= 0) { p.tile = env_pf == 1; p.stream_nb4 = env_pf == 0; }
     const long active = s->E < P ? s->E : P;       // upper bound of experts with rows
     const long slots = 512;                        // 256 CUs x 2 workgroups
     const int G_gu = s->H / ODSD_GROUP, G_dn = s->I / ODSD_GROUP;
@@ -511,9 +510,8 @@ static ExpertsPlan experts_plan(const odsd_moe_shape *s) {
         if (p.MB <= 4) {
             const long wg_gu = active * ((2 * s->I / 16 + 15) / 16);
             if (wg_gu < 4 * slots) p.NB = 2;
-            if (env_nb == 2 || env_nb == 4) p.NB = env_nb;
         } else {
-            p.NB = p.stream_nb4 ? 4 : 2;
+            p.NB = 2;
         }
         const int nchunks_dn = (s->H / 16 + 4 * p.NB - 1) / (4 * p.NB);
         // up to 4 workgroups per CU with at most 4 token blocks, 2 with 8
@@ -522,8 +520,6 @@ static ExpertsPlan experts_plan(const odsd_moe_shape *s) {
         while (KS * 2 <= G_dn / 2 && active * nchunks_dn * KS < want && KS < 16) KS *= 2;
         p.KS = KS;
     }
-    static const int env_ks = getenv("ODSD_GEMM_KS") ? atoi(getenv("ODSD_GEMM_KS")) : 0;
-    if (env_ks > 0 && env_ks <= G_dn) p.KS = env_ks;
     // every split must own at least one group
     while (p.KS > 1 && ((G_dn + p.KS - 1) / p.KS) * (p.KS - 1) >= G_dn) p.KS--;
     // At prefill shapes the fp32 partials would be 0.5 GB written and read back per layer; fp16
@@ -554,7 +550,8 @@ static void launch_gemm(GemmParams &gp, hipStream_t st) {
     gp.nchunks = (gp.NBLK + (WAVES / WK) * NB - 1) / ((WAVES / WK) * NB);
     gp.n_wg = gp.E * gp.nchunks * gp.KS;
     gp.wg_per_xcd = (gp.n_wg + 7) / 8;
-    w4_gemm_kernel<NB, MB, MODE, DEPTH, NA, WK, DIRECT, OCC, WAVES><<<gp.wg_per_xcd * 8, 64 * WAVES, 0, st>>>(gp);
+    ODSD_LAUNCH(MODE == 0 ? ODSD_KERNEL_GATE_UP : ODSD_KERNEL_DOWN,
+                (w4_gemm_kernel<NB, MB, MODE, DEPTH, NA, WK, DIRECT, OCC, WAVES>), gp.wg_per_xcd * 8, 64 * WAVES, st, gp);
 }
 
 // prefill-shaped tile kernel (experts_prefill.hip)
@@ -577,8 +574,7 @@ static void launch_gemm_plan(const ExpertsPlan &pl, GemmParams &gp, hipStream_t 
         gp.y_f16 = pl.y_f16;
         odsd_launch_gemm_prefill<MODE>(gp, st);
     } else {
-        if (pl.stream_nb4) launch_gemm<4, 8, MODE, 2, 4, 1, false, 1>(gp, st);
-        else launch_gemm<2, 8, MODE, 2, 2, 1, false, 2>(gp, st);
+        launch_gemm<2, 8, MODE, 2, 2, 1, false, 2>(gp, st);
     }
 }
 
@@ -651,13 +647,13 @@ static int launch_combine(const odsd_moe_shape *s, const void *y_, const int32_t
 #define COMBINE_GO(XT, YH, ST)                                                                          \
     do {                                                                                                \
         if (batched)                                                                                    \
-            combine_kernel<XT, YH, ST, 4><<<grid, 256, 0, st>>>(y, idx, w, perm, table, (const XT *)residual, \
-                                                                out_f32, (XT *)out_act, row_ss, s->T, s->H,   \
-                                                                s->K, s->E, pl.KS, P);                        \
+            ODSD_LAUNCH(ODSD_KERNEL_COMBINE, (combine_kernel<XT, YH, ST, 4>), grid, 256, st, y, idx, w, perm, \
+                        table, (const XT *)residual, out_f32, (XT *)out_act, row_ss, s->T, s->H, s->K,  \
+                        s->E, pl.KS, P);                                                                \
         else                                                                                            \
-            combine_kernel<XT, YH, ST, 0><<<grid, 256, 0, st>>>(y, idx, w, perm, table, (const XT *)residual, \
-                                                                out_f32, (XT *)out_act, row_ss, s->T, s->H,   \
-                                                                s->K, s->E, pl.KS, P);                        \
+            ODSD_LAUNCH(ODSD_KERNEL_COMBINE, (combine_kernel<XT, YH, ST, 0>), grid, 256, st, y, idx, w, perm, \
+                        table, (const XT *)residual, out_f32, (XT *)out_act, row_ss, s->T, s->H, s->K,  \
+                        s->E, pl.KS, P);                                                                \
     } while (0)
 #define COMBINE_Y(XT, ST)                          \
     do {                                           \
@@ -686,7 +682,7 @@ extern "C" int odsd_combine(const odsd_moe_shape *s, const void *y, const int32_
 int odsd_launch_experts(const odsd_moe_shape *s, const void *x16, const uint64_t *table, const int32_t *idx,
                         const float *w, const int32_t *counts, const int32_t *offsets, const int32_t *perm,
                         const int32_t *slot_token, const void *residual, float *out_f32, void *out_act,
-                        void *ws, size_t ws_bytes, hipStream_t st, double *row_ss, void *const *events) {
+                        void *ws, size_t ws_bytes, hipStream_t st, double *row_ss) {
     int rc = experts_check(s);
     if (rc != ODSD_OK) return rc;
     if (s->T == 0) return ODSD_OK;
@@ -698,14 +694,9 @@ int odsd_launch_experts(const odsd_moe_shape *s, const void *x16, const uint64_t
     float *y = (float *)((char *)ws + pl.h_bytes);
     rc = odsd_w4_gate_up_silu(s, x16, table, counts, offsets, slot_token, h16, st);
     if (rc != ODSD_OK) return rc;
-    if (events && hipEventRecord((hipEvent_t)events[0], st) != hipSuccess) return ODSD_ERR_LAUNCH;
     rc = odsd_w4_down(s, h16, table, counts, offsets, y, st);
     if (rc != ODSD_OK) return rc;
-    if (events && hipEventRecord((hipEvent_t)events[1], st) != hipSuccess) return ODSD_ERR_LAUNCH;
-    rc = launch_combine(s, y, idx, w, perm, table, residual, out_f32, out_act, row_ss, st);
-    if (rc != ODSD_OK) return rc;
-    if (events && hipEventRecord((hipEvent_t)events[2], st) != hipSuccess) return ODSD_ERR_LAUNCH;
-    return ODSD_OK;
+    return launch_combine(s, y, idx, w, perm, table, residual, out_f32, out_act, row_ss, st);
 }
 
 extern "C" int odsd_experts_w4(const odsd_moe_shape *s, const void *x_f16, const uint64_t *table,

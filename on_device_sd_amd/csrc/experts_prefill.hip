@@ -326,7 +326,8 @@ void odsd_launch_gemm_prefill(GemmParams &gp, hipStream_t st) {
     if (gp.PS < 1) gp.PS = 1;
     gp.n_wg = gp.E * gp.nchunks * gp.KS * gp.PS;
     gp.wg_per_xcd = (gp.n_wg + 7) / 8;
-    w4_gemm_prefill_kernel<MODE, 8><<<gp.wg_per_xcd * 8, 512, 0, st>>>(gp);
+    ODSD_LAUNCH(MODE == 0 ? ODSD_KERNEL_GATE_UP : ODSD_KERNEL_DOWN, (w4_gemm_prefill_kernel<MODE, 8>),
+                gp.wg_per_xcd * 8, 512, st, gp);
 }
 
 template void odsd_launch_gemm_prefill<0>(GemmParams &, hipStream_t);

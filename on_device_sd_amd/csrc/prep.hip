@@ -220,11 +220,11 @@ extern "C" int odsd_rmsnorm(const void *x, const void *weight, int32_t dtype, in
     if (T == 0) return ODSD_OK;
     hipStream_t st = (hipStream_t)stream;
     if (dtype == ODSD_DT_F32)
-        rmsnorm_kernel<float><<<T, 256, 0, st>>>((const float *)x, (const float *)weight, H, (double)eps,
-                                                 (float *)out);
+        ODSD_LAUNCH(ODSD_KERNEL_NORM, rmsnorm_kernel<float>, T, 256, st, (const float *)x, (const float *)weight,
+                    H, (double)eps, (float *)out);
     else if (dtype == ODSD_DT_BF16)
-        rmsnorm_kernel<uint16_t><<<T, 256, 0, st>>>((const uint16_t *)x, (const uint16_t *)weight, H,
-                                                    (double)eps, (uint16_t *)out);
+        ODSD_LAUNCH(ODSD_KERNEL_NORM, rmsnorm_kernel<uint16_t>, T, 256, st, (const uint16_t *)x,
+                    (const uint16_t *)weight, H, (double)eps, (uint16_t *)out);
     else
         return ODSD_ERR_DTYPE;
     ODSD_CHECK_LAUNCH();

@@ -369,13 +369,13 @@ static void launch_partial(const RouterPlan &p, const odsd_moe_shape *s, const v
                            const void *norm_w, float eps) {
     const int n_units = p.TT * p.EG * p.S;
     if (p.S % 4 == 0)
-        router_partial_kernel<XT, NE, true><<<n_units / 4, 256, 0, st>>>(
-            (const XT *)x, (const XT *)gw, partial, (half_t *)x16, s->T, s->H, s->E, p.S, p.EG, n_units,
-            norm_ss, (const XT *)norm_w, (double)eps);
+        ODSD_LAUNCH(ODSD_KERNEL_ROUTER_LOGITS, (router_partial_kernel<XT, NE, true>), n_units / 4, 256, st,
+                    (const XT *)x, (const XT *)gw, partial, (half_t *)x16, s->T, s->H, s->E, p.S, p.EG,
+                    n_units, norm_ss, (const XT *)norm_w, (double)eps);
     else
-        router_partial_kernel<XT, NE, false><<<(n_units + 3) / 4, 256, 0, st>>>(
-            (const XT *)x, (const XT *)gw, partial, (half_t *)x16, s->T, s->H, s->E, p.S, p.EG, n_units,
-            norm_ss, (const XT *)norm_w, (double)eps);
+        ODSD_LAUNCH(ODSD_KERNEL_ROUTER_LOGITS, (router_partial_kernel<XT, NE, false>), (n_units + 3) / 4, 256,
+                    st, (const XT *)x, (const XT *)gw, partial, (half_t *)x16, s->T, s->H, s->E, p.S, p.EG,
+                    n_units, norm_ss, (const XT *)norm_w, (double)eps);
 }
 
 int odsd_launch_router(const odsd_moe_shape *s, const void *x, const void *gate_w, int32_t *idx, float *w,
@@ -408,8 +408,8 @@ int odsd_launch_router(const odsd_moe_shape *s, const void *x, const void *gate_
     ODSD_CHECK_LAUNCH();
     const int S_out = p.S % 4 == 0 ? p.S / 4 : p.S;
 #define TOPK_GO(VV)                                                                                   \
-    router_topk_kernel<VV><<<(s->T + 3) / 4, 256, 0, st>>>(partial, s->T, s->E, s->K, S_out, s->renorm, \
-                                                            idx, w, idx64, logits)
+    ODSD_LAUNCH(ODSD_KERNEL_ROUTER_TOPK, router_topk_kernel<VV>, (s->T + 3) / 4, 256, st,            \
+                (const double *)partial, s->T, s->E, s->K, S_out, s->renorm, idx, w, idx64, logits)
     if (s->E <= 64) TOPK_GO(1);
     else if (s->E <= 128) TOPK_GO(2);
     else if (s->E <= 256) TOPK_GO(4);

@@ -353,6 +353,24 @@ class MoeForwardPlan:
             self.ws.numel(), _stream()), "odsd_moe_forward")
         return MoeOutputs(self.out_f32, oa, self.idx, self.w, self.counts, self.offsets, self.perm)
 
+    def run_events(self, events, x: torch.Tensor, gate_weight: torch.Tensor, table: torch.Tensor,
+                   norm_weight: Optional[torch.Tensor] = None, eps: float = 1e-6,
+                   add_residual: bool = False, out_act: Optional[torch.Tensor] = None,
+                   row_sumsq_in: Optional[torch.Tensor] = None,
+                   row_sumsq_out: Optional[torch.Tensor] = None) -> int:
+        """``run`` with every kernel launch carrying its own start / stop events (``events``: an
+        ``_hip.EventList`` of ``2 * _lib.N_KERNELS`` events; kernel slot k uses events 2k, 2k+1).
+        Returns the bit mask of the slots that were launched; routing outputs are not returned."""
+        lib = _lib.load()
+        oa = out_act if out_act is not None else self.out_act
+        mask = C.c_uint32(0)
+        _lib.check(lib.odsd_moe_forward_events(
+            C.byref(self.shape), x.data_ptr(), _ptr(norm_weight), eps, gate_weight.data_ptr(),
+            table.data_ptr(), 1 if add_residual else 0, _ptr(self.out_f32), _ptr(oa),
+            _ptr(row_sumsq_in), _ptr(row_sumsq_out), self.ws.data_ptr(), self.ws.numel(), _stream(),
+            events.array, C.byref(mask)), "odsd_moe_forward_events")
+        return mask.value
+
 
 def moe_forward(x: torch.Tensor, gate_weight: torch.Tensor, table: torch.Tensor, top_k: int,
                 inter: int, renorm: bool, norm_weight: Optional[torch.Tensor] = None,

@@ -231,12 +231,25 @@ class MoEOnlyStack:
         self.rowss = [ops.row_stats(T, config.hidden_size, self.device) for _ in range(2)]
         self.graph = None
 
-    def _run_layers(self):
+    def _run_layers(self, events=None):
+        masks = []
         for l in range(self.L):
-            self.plan.run(self.buf[l & 1], self.gate[l], self.tables[l], self.norm[l],
-                          self.config.rms_norm_eps, add_residual=True, out_act=self.buf[(l + 1) & 1],
-                          row_sumsq_in=self.rowss[l & 1] if l > 0 else None,
-                          row_sumsq_out=self.rowss[(l + 1) & 1] if l + 1 < self.L else None)
+            kw = dict(add_residual=True, out_act=self.buf[(l + 1) & 1],
+                      row_sumsq_in=self.rowss[l & 1] if l > 0 else None,
+                      row_sumsq_out=self.rowss[(l + 1) & 1] if l + 1 < self.L else None)
+            if events is None:
+                self.plan.run(self.buf[l & 1], self.gate[l], self.tables[l], self.norm[l],
+                              self.config.rms_norm_eps, **kw)
+            else:
+                masks.append(self.plan.run_events(events[l], self.buf[l & 1], self.gate[l], self.tables[l],
+                                                  self.norm[l], self.config.rms_norm_eps, **kw))
+        return masks
+
+    def forward_events(self, hidden: torch.Tensor, events):
+        """``forward`` (eager) with the kernels of layer l timed by the events ``events[l]``
+        (see ``MoeForwardPlan.run_events``); returns the launched-slot mask of every layer."""
+        self.buf[0].copy_(hidden)
+        return self._run_layers(events)
 
     def capture(self):
         """Record the stack into a HIP graph (all kernels, no memset nodes)."""

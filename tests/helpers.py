@@ -49,3 +49,16 @@ def check_output(got: torch.Tensor, ref: torch.Tensor, rows=None):
     assert mx <= MAX_ABS_TOL, f"max-abs error {mx:.4e} > {MAX_ABS_TOL}"
     assert mean <= MEAN_ABS_TOL, f"mean-abs error {mean:.4e} > {MEAN_ABS_TOL}"
     return mx, mean
+
+
+def check_output_relative(got: torch.Tensor, ref: torch.Tensor, max_rel: float = 1e-2, mean_rel: float = 2e-3):
+    """max|err| <= max_rel * max|ref| and mean|err| <= mean_rel * mean|ref|: the error held against
+    the reference's own scale (the absolute tolerances of check_output are 100-1000 times the
+    size of small test outputs)."""
+    got = got.detach().float().cpu()
+    err = (got - ref).abs()
+    mx = err.max().item() / max(ref.abs().max().item(), 1e-30)
+    mean = err.mean().item() / max(ref.abs().mean().item(), 1e-30)
+    assert mx <= max_rel, f"max error is {mx:.3e} of max|ref| (> {max_rel})"
+    assert mean <= mean_rel, f"mean error is {mean:.3e} of mean|ref| (> {mean_rel})"
+    return mx, mean

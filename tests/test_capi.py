@@ -90,3 +90,7 @@ def test_static_scratch_call_refuses_what_does_not_fit():
     text = open(os.path.join(ROOT, "include", "odsd_moe.h")).read()
     m = re.search(r"#define ODSD_STATIC_SCRATCH_BYTES \((\d+)u << (\d+)\)", text)
     assert m and int(m.group(1)) << int(m.group(2)) == _lib.STATIC_SCRATCH_BYTES
+    # the events form needs its event array
+    ok = _lib.MoeShape(8, 256, 8, 2, 256, 1, _lib.DT_BF16, 0)
+    assert lib.odsd_moe_forward_events(C.byref(ok), 1 << 20, None, 1e-6, 1 << 20, 1 << 20, 0, 1 << 20, None,
+                                       None, None, 1 << 20, 1 << 30, None, None, None) == 1

@@ -4,7 +4,7 @@ import pytest
 import torch
 
 from oracle import moe_oracle as orc
-from tests.helpers import canon_to_oracle, check_output
+from tests.helpers import canon_to_oracle, check_output, check_output_relative
 
 pytestmark = pytest.mark.gpu
 
@@ -176,15 +176,16 @@ def test_dispatch_duplicates_and_out_of_range(dev):
     assert np.array_equal(d.inv.cpu().numpy(), inv)
 
 
-def _small_layer(dev, T, H, E, K, I, dtype, seed, renorm=True):
+def _small_layer(dev, T, H, E, K, I, dtype, seed, renorm=True, w_mean=0.0, w_std=0.02):
+    """Expert weights N(w_mean, w_std): a non-zero mean gives every group a large zero point."""
     import on_device_sd_amd as odsd
     g = torch.Generator().manual_seed(seed)
     wg = (torch.randn(E, H, generator=g) * 0.02).to(dtype)
     bank = odsd.W4ExpertBank(E, H, I, dev)
     experts = {}
+    mk = lambda n, k: torch.randn(n, k, generator=g) * w_std + w_mean
     for e in range(E):
-        canon = bank.load_expert(e, torch.randn(I, H, generator=g) * 0.02, torch.randn(I, H, generator=g) * 0.02,
-                                 torch.randn(H, I, generator=g) * 0.02, keep_canonical=True)
+        canon = bank.load_expert(e, mk(I, H), mk(I, H), mk(H, I), keep_canonical=True)
         experts[e] = canon_to_oracle(canon)
     x = torch.randn(T, H, generator=g).to(dtype)
     return wg, bank, experts, x
@@ -230,11 +231,68 @@ def test_moe_forward_vs_oracle(dev, T, H, E, K, I, dtype):
     assert np.array_equal(out.perm.cpu().numpy(), perm)
     mx, mean = check_output(out.out_f32, ref)
     print(f"  max-abs {mx:.3e} mean-abs {mean:.3e}", flush=True)
+    # the outer tolerances are absolute and these outputs are small: hold the kernel to the
+    # reference's own scale as well, so that a dropped tail block or a few wrong rows cannot pass
+    check_output_relative(out.out_f32, ref)
     # the activation-dtype output is the fp32 one rounded once
     assert torch.equal(out.out_act.cpu(), out.out_f32.cpu().to(dtype))
     # determinism: a second run gives the same bits
     out2 = ops.moe_forward(x.to(dev), wg.to(dev), bank.table(), K, I, renorm=True)
     assert torch.equal(out2.out_f32, out.out_f32)
+
+
+# weights whose groups sit far from zero: |zero point| of tens to hundreds, |w| ~ 0.3 .. 0.5
+OFFSET_CASES = [
+    # T, H, E, K, I, w_mean, w_std
+    (40, 512, 4, 2, 384, 0.3, 0.02),
+    (40, 512, 4, 2, 384, -0.5, 0.01),
+    (6, 1024, 4, 2, 256, 0.3, 0.02),        # direct path
+    (600, 256, 2, 2, 384, 0.15, 0.01),      # tile kernel (fp16 y: keep the outputs inside fp16 range)
+]
+
+
+@pytest.mark.parametrize("T,H,E,K,I,w_mean,w_std", OFFSET_CASES)
+def test_moe_forward_offset_weight_groups(dev, T, H, E, K, I, w_mean, w_std):
+    """Non-zero-mean weight groups: the zero-point term (scale*zero times the group sums of the
+    activations) is large against the code term, so an error in it shows."""
+    print("moe_forward offset weights", T, H, E, K, I, w_mean, w_std, flush=True)
+    ops = _ops()
+    wg, bank, experts, x = _small_layer(dev, T, H, E, K, I, torch.bfloat16, seed=T + I, w_mean=w_mean, w_std=w_std)
+    zmax = max(float(np.abs(ex.gate[2].astype(np.float32)).max()) for ex in experts.values())
+    assert zmax > 10.0, "the case is meant to have large zero points"
+    out = ops.moe_forward(x.to(dev), wg.to(dev), bank.table(), K, I, renorm=True)
+    ref, idx, w = orc.moe_block(x, wg, experts, K, True)
+    assert np.array_equal(out.idx.cpu().numpy(), idx)
+    mx, mean = check_output_relative(out.out_f32, ref, max_rel=2e-3, mean_rel=2e-4)
+    print(f"  relative to max|ref|: max {mx:.3e}; mean error / mean|ref| {mean:.3e}", flush=True)
+
+
+@pytest.mark.parametrize("T,H,E,K,I,dtype", [c for i, c in enumerate(EXPERT_CASES) if i in (0, 2, 4, 8, 11, 13, 17)])
+def test_gate_up_h_rows(dev, T, H, E, K, I, dtype):
+    """The gate_up stage alone: h = silu(x Wg^T) * (x Wu^T) per dispatched pair against the
+    oracle's dequantised weights."""
+    print("gate_up h rows", T, H, E, K, I, dtype, flush=True)
+    ops = _ops()
+    wg, bank, experts, x = _small_layer(dev, T, H, E, K, I, dtype, seed=T + H)
+    idx, w, _, x16 = ops.router_topk(x.to(dev), wg.to(dev), K, True, want_f16=True)
+    disp = ops.dispatch(idx, E)
+    st = ops.ExpertStages(T, H, E, K, I, dtype, dev)
+    st.h16.fill_(float("nan"))
+    h = st.gate_up(x16, bank.table(), disp).cpu()
+    torch.cuda.synchronize()
+    assert h.shape == (T * K, I) and torch.isfinite(h).all()
+    slot_token = disp.slot_token.cpu().numpy()
+    offs = disp.offsets.cpu().numpy()
+    x32 = x.to(torch.float16).to(torch.float32)
+    for e in range(E):
+        rows = slot_token[offs[e]:offs[e + 1]]
+        if len(rows) == 0:
+            continue
+        gw, uw, _ = experts[e].dequant()
+        ref = torch.nn.functional.silu(x32[rows] @ gw.T) * (x32[rows] @ uw.T)
+        got = h[offs[e]:offs[e + 1], :I].to(torch.float32)
+        err = (got - ref).abs().max().item()
+        assert err <= 2e-3 * max(ref.abs().max().item(), 1e-3) + 1e-4, (e, err)
 
 
 @pytest.mark.gpu
