@@ -22,6 +22,8 @@
 // and the indexed "+=" combine (:363, :376).
 #include "w4_gemm.h"
 
+#include <type_traits>
+
 // NB    16-row weight blocks per wavefront          MB  16-row token blocks per pass
 // DEPTH groups of weight loads kept in flight       NA  blocks expanded to fp16 at a time
 // WK    wavefronts of a workgroup that split the reduction dimension among themselves
@@ -162,17 +164,6 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
                 if (DIRECT) {
                     wq[buf][i] = __builtin_nontemporal_load((const global_u4 *)(qp_c + (wq_off[i] + gc * 1024u)));
                     wsz[buf][i] = *(const global_u32 *)(szp_c + (sz_off[i] + gc * 64u));
-                } else if (MODE == 1) {
-                    // The ring refills past the last group are still issued (the loop body is
-                    // branch-free).  The down projection's reductions are short (6 groups at I = 768,
-                    // so 2 refills in 8 loads would be wasted): there they go to an offset outside
-                    // the buffer, which returns zeros without touching memory (the range check of a
-                    // raw buffer looks at the per-lane offset only), where a clamped address reads
-                    // the last tile again.  At the cost of a select per load; with the long
-                    // reductions of gate_up the select costs more than the few tiles it saves.
-                    const bool live = g < g_end;
-                    wq[buf][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_q, (int)(live ? wq_off[i] : 0xFFFFFFF0u), (int)(gc * 1024u), 2 /* nt */);
-                    wsz[buf][i] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_sz, (int)(live ? sz_off[i] : 0xFFFFFFF0u), (int)(gc * 64u), 0);
                 } else {
                     wq[buf][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_q, (int)wq_off[i], (int)(gc * 1024u), 2 /* nt */);
                     wsz[buf][i] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_sz, (int)sz_off[i], (int)(gc * 64u), 0);
@@ -195,7 +186,7 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
             for (int i = 0; i < XPT; ++i) {
                 // piece i covers ROWS_PER_PIECE rows from row ROWS_PER_PIECE * i on: nothing to
                 // fetch for a token block without rows
-                if (i * ROWS_PER_PIECE < mcnt_s && (MODE == 0 || g < g_end)) {
+                if (i * ROWS_PER_PIECE < mcnt_s) {
                     lds_void *dst = (lds_void *)(xs_raw + buf * (16 * MB * 256) + (i * 64 * WAVES + wave * 64) * 16);
                     dma16_to_lds(xg, st_off[i], dst);
                 }
@@ -217,73 +208,95 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
             __builtin_amdgcn_s_barrier();
         }
 
-        int it = 0;
-        for (int g = g_begin; g < g_end;) {
-            // The step loop is unrolled over several trips round the ring: at a loop header the
-            // compiler's wait-count bookkeeping falls back to draining every outstanding load
-            // before the first use of ring data, so the fewer headers the stream crosses, the
-            // less often the prefetch pipeline runs empty.
+        // One step = one group: expand ring slot d, refill it with group g + DEPTH, multiply.
+        // REFILL is a compile-time flag: the last DEPTH groups of the reduction have nothing left
+        // to fetch, and their steps are compiled without the refill (a refill clamped to the
+        // last group would read that tile again: DEPTH of G tiles per block, 12 % of the stream
+        // at G = 16, a third at G = 6).
+        auto step = [&](auto refill_c, const int d, const int xb, const int g) {
+            constexpr bool REFILL = decltype(refill_c)::value;
+            // issue order is pinned: as soon as this slot's codes have been expanded, the DMA
+            // of the next group's token rows (into the buffer the previous step read; every
+            // wavefront has passed that step's barrier) and the slot's refill, then the products.
+            // (The compiler cannot see the DMA loads.  Issued after the expansion, the vmcnt
+            // wait it derives for the slot retires exactly the slot and the previous DMA.)
+            half8_t bdir[4];
+            if (DIRECT) {
 #pragma unroll
-            for (int u = 0; u < DEPTH * RING_TRIPS; ++u) {
-                const int d = u % DEPTH;
-                // issue order is pinned: as soon as this slot's codes have been expanded, the DMA
-                // of the next group's token rows (into the buffer the previous step read; every
-                // wavefront has passed that step's barrier) and the slot's refill, then the products.
-                // (The compiler cannot see the DMA loads.  Issued after the expansion, the vmcnt
-                // wait it derives for the slot retires exactly the slot and the previous DMA.)
-                // with an even number of steps per trip the token buffer of a step is known at
-                // compile time (every trip starts on an even step) and becomes an immediate offset
-                const int xb = (DEPTH * RING_TRIPS) % 2 == 0 ? (u & 1) : (it & 1);
-                half8_t bdir[4];
-                if (DIRECT) {
+                for (int j = 0; j < 4; ++j) bdir[j] = __builtin_bit_cast(half8_t, xd[DIRECT ? d : 0][j]);
+            }
+            // this step's token buffer: one add per 32-column step, the block is an immediate
+            const char *xfrag[4];
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) bdir[j] = __builtin_bit_cast(half8_t, xd[DIRECT ? d : 0][j]);
+            for (int j = 0; j < 4; ++j) xfrag[j] = xs_raw + (uint32_t)(xb * (16 * MB * 256)) + lds_frag[j];
+            const int nmb_s = DIRECT ? nmb : scalar_int(nmb);
+#pragma unroll
+            for (int h = 0; h < NB; h += NA) {
+                half8_t a[NA][4];
+#pragma unroll
+                for (int i = 0; i < NA; ++i) dequant_tile(dc, wq[d][h + i], wsz[d][h + i], a[i]);
+                if (h + NA >= NB) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (!DIRECT && (REFILL || g + 1 < g_end)) dma_x(xb ^ 1, g + 1);
+                    if (REFILL) load_w(d, g + DEPTH);      // ring slot d is free again
+                    __builtin_amdgcn_sched_barrier(0);
                 }
-                // this step's token buffer: one add per 32-column step, the block is an immediate
-                const char *xfrag[4];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) xfrag[j] = xs_raw + (uint32_t)(xb * (16 * MB * 256)) + lds_frag[j];
-                const int nmb_s = DIRECT ? nmb : scalar_int(nmb);
+                for (int m = 0; m < MB; ++m) {
+                    if (m < nmb_s) {
 #pragma unroll
-                for (int h = 0; h < NB; h += NA) {
-                    half8_t a[NA][4];
+                        for (int j = 0; j < 4; ++j) {
+                            half8_t bx;
+                            if (DIRECT) bx = bdir[j];
+                            else bx = *(const half8_t *)(xfrag[j] + m * 4096);
 #pragma unroll
-                    for (int i = 0; i < NA; ++i) dequant_tile(dc, wq[d][h + i], wsz[d][h + i], a[i]);
-                    if (h + NA >= NB) {
-                        __builtin_amdgcn_sched_barrier(0);
-                        if (!DIRECT) dma_x(xb ^ 1, g + 1);
-                        load_w(d, g + DEPTH);      // ring slot d is free again
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-#pragma unroll
-                    for (int m = 0; m < MB; ++m) {
-                        if (m < nmb_s) {
-#pragma unroll
-                            for (int j = 0; j < 4; ++j) {
-                                half8_t bx;
-                                if (DIRECT) bx = bdir[j];
-                                else bx = *(const half8_t *)(xfrag[j] + m * 4096);
-#pragma unroll
-                                for (int i = 0; i < NA; ++i)
-                                    acc[h + i][m] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i][j], bx, acc[h + i][m], 0, 0, 0);
-                            }
+                            for (int i = 0; i < NA; ++i)
+                                acc[h + i][m] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i][j], bx, acc[h + i][m], 0, 0, 0);
                         }
                     }
                 }
-                if (DIRECT) {
-                    __builtin_amdgcn_sched_barrier(0);
-                    load_xd(d, g + DEPTH);
-                } else {
-                    __builtin_amdgcn_sched_barrier(0);
-                    // x(g+1) was issued in this step, before this step's refill: once only the
-                    // refill is outstanding it has landed (and so has the previous step's refill,
-                    // which the next step starts with anyway)
-                    ODSD_WAIT_VMCNT(2 * NB);
-                    __builtin_amdgcn_s_barrier();
+            }
+            if (DIRECT) {
+                __builtin_amdgcn_sched_barrier(0);
+                if (REFILL) load_xd(d, g + DEPTH);
+            } else {
+                __builtin_amdgcn_sched_barrier(0);
+                // x(g+1) was issued in this step, before this step's refill: once only the
+                // refill is outstanding it has landed (and so has the previous step's refill,
+                // which the next step starts with anyway)
+                if (REFILL) ODSD_WAIT_VMCNT(2 * NB);
+                else ODSD_WAIT_VMCNT(0);
+                __builtin_amdgcn_s_barrier();
+            }
+        };
+        // with an even number of steps per trip the token buffer of a step is known at compile
+        // time (every trip starts on an even step) and becomes an immediate offset
+        constexpr bool XB_STATIC = DEPTH % 2 == 0;
+        int it = 0, g = g_begin;
+        // Main part: whole trips round the ring while more than DEPTH groups remain (a trip whose
+        // later refills run past the last group clamps them: at most DEPTH - 1 tiles per block).
+        // Several trips per loop iteration: at a loop header the compiler's wait-count
+        // bookkeeping falls back to draining every outstanding load before the first use of ring
+        // data, so the fewer headers the stream crosses, the less often the pipeline runs empty.
+        while (g + DEPTH < g_end) {
+#pragma unroll
+            for (int t = 0; t < RING_TRIPS; ++t) {
+#pragma unroll
+                for (int d = 0; d < DEPTH; ++d) {
+                    step(std::true_type{}, d, XB_STATIC ? (d & 1) : (it & 1), g);
+                    ++g;
+                    ++it;
                 }
+                if (!(g + DEPTH < g_end)) break;
+            }
+        }
+        // Tail: the groups that are already in the ring.
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            if (g < g_end) {
+                step(std::false_type{}, d, XB_STATIC ? (d & 1) : (it & 1), g);
                 ++g;
                 ++it;
-                if (g >= g_end) break;
             }
         }
 
