@@ -107,14 +107,15 @@ class W4MoERunner:
         return LayerOutput(hidden_states=out, metadata=meta)
 
     # -- internals -----------------------------------------------------------------------------
-    def _placement_table(self, placement: ExpertPlacement) -> torch.Tensor:
+    def _placement_table(self, placement: ExpertPlacement, only: Optional[frozenset] = None) -> torch.Tensor:
         """Device pointer table of a placement.  Placements repeat from step to step, so tables
         are cached; the key is built from the identities of the parameter objects (a bank hands
         out one object per expert), and the cache entry keeps those objects alive so that an
-        identity cannot be reused while the entry exists."""
+        identity cannot be reused while the entry exists.  ``only``: expert ids that may execute
+        (the activated set of a hand-built routing result); the rows of all others stay empty."""
         gpu, cpu, sub = placement.gpu_expert_params, placement.cpu_expert_params, placement.substitution_map
         key = (tuple(gpu), tuple(map(id, gpu.values())), tuple(cpu), tuple(map(id, cpu.values())),
-               tuple(sub.items()) if sub else ())
+               tuple(sub.items()) if sub else (), only)
         hit = self._table_cache.get(key)
         if hit is not None:
             for p in hit[2]:             # bundles of cache pools only (usually none)
@@ -132,7 +133,7 @@ class W4MoERunner:
                 params[e] = p
         if len(self._table_cache) > 64:
             self._table_cache.clear()
-        tab = build_table(self.config.num_experts, params, sub, self.device)
+        tab = build_table(self.config.num_experts, params, sub, self.device, only=only)
         held = list(gpu.values()) + list(cpu.values())
         self._table_cache[key] = (tab, held, [p for p in held if p.bank.recycles])
         return tab
@@ -155,7 +156,14 @@ class W4MoERunner:
             idx = disp.idx32          # the router's own int32 indices: no conversion kernel
         scores = routing.topk_scores.reshape(flat.shape[0], -1).to(device=flat.device,
                                                                   dtype=torch.float32)
-        table = self._placement_table(placement)
+        # The reference executes the experts listed in activated_expert_ids and nothing else
+        # (qwen3_runner.py:303).  route_experts returns exactly the set of selected experts, so a
+        # routing result that carries its device-side dispatch needs no check; a hand-built one
+        # may list a subset, and the pairs of every expert outside it contribute nothing.
+        only = None
+        if routing.dispatch is None:
+            only = frozenset(e.expert_idx for e in routing.activated_expert_ids)
+        table = self._placement_table(placement, only)
         # the fp16 copy the router wrote, if these are the very hidden states it routed
         x16 = routing.x_f16 if routing.x_f16 is not None and routing.x_tag == _tensor_tag(flat) \
             else ops.to_f16(flat)

@@ -175,13 +175,17 @@ class W4ExpertBank:
 
 
 def build_table(num_experts: int, params: Dict[int, W4ExpertParams],
-                substitution: Optional[Dict[int, int]] = None, device="cuda") -> torch.Tensor:
+                substitution: Optional[Dict[int, int]] = None, device="cuda",
+                only: Optional[Iterable[int]] = None) -> torch.Tensor:
     """Pointer table for an arbitrary placement: row e points at params[e], or at
-    params[substitution[e]], or is 0 (expert skipped)."""
+    params[substitution[e]], or is 0 (expert skipped).  With ``only``, experts outside that
+    set are skipped whatever the placement holds for them."""
     substitution = substitution or {}
     rows = []
     for e in range(num_experts):
         src = e if e in params else substitution.get(e)
+        if only is not None and e not in only:
+            src = None
         if src is not None and src in params:
             p = params[src]
             if not isinstance(p, W4ExpertParams):

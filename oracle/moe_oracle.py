@@ -131,7 +131,21 @@ def unpack_codes(q: np.ndarray) -> np.ndarray:
 
 
 def dequantize_w4(q: np.ndarray, scale: np.ndarray, zero: np.ndarray) -> np.ndarray:
-    """deq = (q - zero) * scale in fp32 (quant.py:106), per group."""
+    """deq = (q - zero) * scale in fp32 (quant.py:106), per group.  Evaluated with torch's CPU
+    elementwise kernels (multi-threaded; the same two correctly rounded fp32 operations as the
+    numpy form below, which a test holds it equal to bit for bit)."""
+    qt = torch.from_numpy(np.ascontiguousarray(q))
+    n, kb = qt.shape
+    kd = kb * 2
+    g = kd // GROUP
+    codes = torch.stack((qt & 0x0F, qt >> 4), dim=-1).view(n, kd).to(torch.float32)
+    zf = torch.from_numpy(np.ascontiguousarray(zero)).to(torch.float32)[:, :, None]
+    sf = torch.from_numpy(np.ascontiguousarray(scale)).to(torch.float32)[:, :, None]
+    return ((codes.view(n, g, GROUP) - zf) * sf).view(n, kd).numpy()
+
+
+def dequantize_w4_numpy(q: np.ndarray, scale: np.ndarray, zero: np.ndarray) -> np.ndarray:
+    """The same in plain numpy (slow; kept as the statement dequantize_w4 is checked against)."""
     codes = unpack_codes(q).astype(np.float32)
     n, kd = codes.shape
     g = kd // GROUP

@@ -106,6 +106,27 @@ def test_substitution_uses_substitute_params(runner, dev):
     assert out.abs().sum() > 0
 
 
+def test_activated_subset_of_a_hand_built_routing_result(runner, dev):
+    """The reference loops over routing.activated_expert_ids (qwen3_runner.py:303): a hand-built
+    RoutingResult whose set is a strict subset of the selected experts executes only that subset
+    (the reference's own tests build such results, demo/tests/unit/test_forward_moe.py:53)."""
+    import on_device_sd_amd as odsd
+    hidden = _hidden(dev, 4, H, seed=21)
+    idx = torch.tensor([[0, 1], [1, 2], [2, 3], [3, 0]], device=dev)
+    scores = torch.full(idx.shape, 0.5, dtype=torch.float32, device=dev)
+    params = runner.banks[0].all_expert_params()
+    rr = odsd.RoutingResult(layer_idx=0, topk_indices=idx, topk_scores=scores,
+                            activated_expert_ids={odsd.ExpertID(0, 1), odsd.ExpertID(0, 3)})
+    placement = odsd.ExpertPlacement(gpu_expert_params=params, cpu_expert_params={}, routing_result=rr)
+    out = runner._execute_moe_with_placement(hidden, placement)
+    ref = orc.moe_forward(hidden.cpu(), idx.cpu().numpy(), scores.cpu().numpy(),
+                          {e: x for e, x in runner.oracle_experts[0].items() if e in (1, 3)})
+    check_output(out, ref)
+    full = runner._execute_moe_with_placement(hidden, odsd.ExpertPlacement(
+        gpu_expert_params=params, cpu_expert_params={}, routing_result=_routing(0, idx, scores)))
+    assert (full.float() - out.float()).abs().max() > 1e-3     # the skipped experts do matter here
+
+
 def test_four_pairs_per_token_with_absent_and_repeated_experts(runner, dev):
     """K = 4 takes the combine's batched row fetch; pairs of an expert that is not placed are
     skipped there without their rows being used."""

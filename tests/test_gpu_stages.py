@@ -295,6 +295,71 @@ def test_gate_up_h_rows(dev, T, H, E, K, I, dtype):
         assert err <= 2e-3 * max(ref.abs().max().item(), 1e-3) + 1e-4, (e, err)
 
 
+def _clamped_reference(x, idx, w, experts, lim=65504.0):
+    """The oracle's per-expert loop with the two places where the device path holds fp16 values
+    made explicit: activations and h = silu(g) * u are clamped to +-65504."""
+    xf = x.to(torch.float32).clamp(-lim, lim)
+    T, K = idx.shape
+    out = torch.zeros(T, xf.shape[1])
+    for k in range(K):
+        for t in range(T):
+            gw, uw, dw = experts[int(idx[t, k])].dequant()
+            h = (torch.nn.functional.silu(xf[t] @ gw.T) * (xf[t] @ uw.T)).clamp(-lim, lim)
+            out[t] += float(w[t, k]) * (h @ dw.T)
+    return out
+
+
+def test_outlier_activations(dev):
+    """bf16 activations with outliers.  Up to a few thousand (far beyond what LLM residual
+    streams hold) the block stays within the relative tolerance of the fp32 reference.  Past the
+    fp16 range the path saturates instead of overflowing: activations above 65504 and
+    intermediate h values above 65504 are clamped, and the result is the reference evaluated with
+    exactly those two clamps -- finite, deterministic, and different from the unclamped
+    reference, which is the documented limit of the fp16 operand format."""
+    print("outlier activations", flush=True)
+    ops = _ops()
+    T, H, E, K, I = 12, 512, 4, 2, 256
+    wg, bank, experts, x = _small_layer(dev, T, H, E, K, I, torch.bfloat16, seed=77)
+    experts = {e: tuple(ex.dequant()) for e, ex in experts.items()}
+
+    class _E:            # pre-dequantised experts with the W4Expert interface the helper uses
+        def __init__(self, t): self.t = t
+        def dequant(self): return self.t
+    experts_c = {e: _E(t) for e, t in experts.items()}
+    # (a) outliers of a few thousand: in tolerance against the plain oracle
+    xa = x.clone()
+    xa[1, 7], xa[3, 100], xa[5, 300], xa[8, 511] = 3000.0, -3000.0, 2500.0, -1800.0
+    out = ops.moe_forward(xa.to(dev), wg.to(dev), bank.table(), K, I, renorm=True)
+    ref, idx, w = orc.moe_block(xa, wg, experts, K, True)
+    assert np.array_equal(out.idx.cpu().numpy(), idx)
+    mx, mean = check_output_relative(out.out_f32, ref, max_rel=2e-3, mean_rel=1e-3)
+    print(f"  outliers to 3e3: max error {mx:.2e} of max|ref| = {ref.abs().max().item():.1f}", flush=True)
+    # (b) entries at +-3e4 and one beyond fp16: saturation, equal to the clamped reference
+    xb = x.clone()
+    xb[0, 3], xb[2, 50], xb[4, 200] = 3.0e4, -3.0e4, 1.0e5
+    out = ops.moe_forward(xb.to(dev), wg.to(dev), bank.table(), K, I, renorm=True)
+    assert torch.isfinite(out.out_f32).all()
+    lg = orc.router_logits(xb, wg)                      # routing sees the unclamped activations
+    idx, w = orc.route(lg, K, True)
+    assert np.array_equal(out.idx.cpu().numpy(), idx)
+    ref_c = _clamped_reference(xb, idx, w, experts_c)
+    mx, mean = check_output_relative(out.out_f32, ref_c, max_rel=2e-3, mean_rel=1e-3)
+    ref_u = orc.moe_forward(xb, idx, w, experts)
+    assert (ref_u - ref_c).abs().max() > 1.0, "the case is meant to reach the clamps"
+    print(f"  saturating inputs: max error {mx:.2e} of max|clamped ref| = {ref_c.abs().max().item():.3e}", flush=True)
+
+
+def test_bank_unpacks_to_the_canonical_arrays(dev):
+    """The packed bytes a bank holds decode, through the oracle's inverse of the layout, to the
+    canonical (codes, scale, zero) the quantiser produced."""
+    from tests.helpers import unpack_bank_expert
+    wg, bank, experts, x = _small_layer(dev, 4, 256, 3, 1, 384, torch.bfloat16, seed=5)
+    for e in range(3):
+        got = unpack_bank_expert(bank, e)
+        for a, b in zip((got.gate, got.up, got.down), (experts[e].gate, experts[e].up, experts[e].down)):
+            assert all(np.array_equal(np.asarray(u).view(np.uint8), np.asarray(v).view(np.uint8)) for u, v in zip(a, b))
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("H", [128, 1280, 2048])
 def test_rmsnorm_folded_into_router_matches_standalone(dev, H):

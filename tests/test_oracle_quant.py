@@ -89,3 +89,11 @@ def test_pack_layout_bruteforce(stride, offset):
     assert not qp[other].any()
     q2, s2, z2 = orc.unpack_w4(qp, sz, stride, offset)
     assert np.array_equal(q2, q) and np.array_equal(s2, s) and np.array_equal(z2, z)
+
+
+def test_fast_dequant_equals_the_numpy_statement():
+    rng = np.random.default_rng(9)
+    w = (rng.standard_normal((48, 640)) * 0.05 + rng.standard_normal((48, 1)) * 0.2).astype(np.float32)
+    q, s, z = orc.quantize_w4(w)
+    a, b = orc.dequantize_w4(q, s, z), orc.dequantize_w4_numpy(q, s, z)
+    assert a.dtype == np.float32 and np.array_equal(a.view(np.uint32), b.view(np.uint32))
