@@ -33,7 +33,9 @@ class RoutingResult:
     route_experts already produced; forward_moe recomputes them when it is absent
     (for example on a hand-built RoutingResult).  ``x_f16`` is the fp16 copy of the routed
     hidden states that the router kernel writes anyway, tagged with the identity of the tensor
-    it was made from; forward_moe uses it when it is handed that same, unmodified tensor.
+    it was made from; forward_moe uses it when it is handed that same, unmodified tensor
+    (unmodified as far as torch's version counter tells: a caller that overwrites the routed
+    tensor in place through something other than torch must clear ``x_f16``).
     """
     layer_idx: int
     topk_indices: torch.Tensor
@@ -42,6 +44,9 @@ class RoutingResult:
     dispatch: Optional[Any] = field(default=None, repr=False, compare=False)
     x_f16: Optional[torch.Tensor] = field(default=None, repr=False, compare=False)
     x_tag: Optional[Tuple] = field(default=None, repr=False, compare=False)
+    # the routed tensor itself: while the routing result lives, its storage cannot be handed to
+    # another tensor, so the address in x_tag keeps meaning "that tensor"
+    x_src: Optional[torch.Tensor] = field(default=None, repr=False, compare=False)
 
     @property
     def top_k(self) -> int:

@@ -371,14 +371,16 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
                                                       const XT *__restrict__ residual,
                                                       float *__restrict__ out_f32, XT *__restrict__ out_act,
                                                       double *__restrict__ row_ss,
-                                                      int T, int H, int K, int E, int KS, int P) {
+                                                      int T, int H, int K, int E, int KS, int P, int nchunk) {
     // One workgroup per (token, 1024-column chunk).  STATS: it also leaves the sum of squares of
     // what it stored in out_act, row_ss[t][chunk] -- the statistic the next block's RMSNorm
     // starts from (chunk sums are added in ascending order by whoever consumes them).
-    const int t = blockIdx.y;
+    // (token and chunk share the x dimension of the grid: the y dimension ends at 65535)
+    const int t = blockIdx.x / nchunk;
+    const int chunk = blockIdx.x - t * nchunk;
     double ss = 0.0;
     {
-        const int c = (blockIdx.x * 256 + threadIdx.x) * 4;
+        const int c = (chunk * 256 + threadIdx.x) * 4;
         if (c < H) {
         float4_t acc = {0.f, 0.f, 0.f, 0.f};
         if (KB > 0) {
@@ -462,7 +464,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
         ss = wave_sum(ss);
         if (lane_id() == 0) red[threadIdx.x >> 6] = ss;
         __syncthreads();
-        if (threadIdx.x == 0) row_ss[(size_t)t * gridDim.x + blockIdx.x] = (red[0] + red[1]) + (red[2] + red[3]);
+        if (threadIdx.x == 0) row_ss[(size_t)t * nchunk + chunk] = (red[0] + red[1]) + (red[2] + red[3]);
     }
 }
 
@@ -549,6 +551,13 @@ static int experts_check(const odsd_moe_shape *s) {
     if (s->H % ODSD_GROUP || s->I % ODSD_GROUP) return ODSD_ERR_SHAPE;
     if ((int64_t)s->T * s->K > 0x7fffffffLL) return ODSD_ERR_SHAPE;
     if (s->act_dtype != ODSD_DT_F32 && s->act_dtype != ODSD_DT_BF16) return ODSD_ERR_DTYPE;
+    // the kernels address token rows and weight tiles with 32-bit byte offsets: a row of x is
+    // found at token * H * 2, a row of h at slot * I * 2, a tile inside one expert's matrix
+    const int64_t P = (int64_t)s->T * s->K;
+    const int64_t hi = s->H > s->I ? s->H : s->I;
+    if ((int64_t)s->T * s->H * 2 >= (1LL << 32) || P * s->I * 2 >= (1LL << 32) || P * hi * 2 >= (1LL << 32))
+        return ODSD_ERR_UNSUPPORTED;
+    if ((int64_t)s->H * s->I >= (1LL << 31)) return ODSD_ERR_UNSUPPORTED;   // 2 I x H / 2 bytes of codes
     return ODSD_OK;
 }
 
@@ -652,21 +661,22 @@ static int launch_combine(const odsd_moe_shape *s, const void *y_, const int32_t
     if (!out_f32 && !out_act) return ODSD_ERR_NULL;
     if (row_ss && !out_act) return ODSD_ERR_NULL;
     if (!odsd_aligned16(y) || (out_f32 && !odsd_aligned16(out_f32))) return ODSD_ERR_ALIGN;
-    if (s->T > 65535) return ODSD_ERR_UNSUPPORTED;
     const ExpertsPlan pl = experts_plan(s);
     const int P = s->T * s->K;
-    const dim3 grid((s->H / 4 + 255) / 256, s->T);
+    const int nchunk = (s->H / 4 + 255) / 256;
+    if ((int64_t)nchunk * s->T > 0x7fffffffLL) return ODSD_ERR_UNSUPPORTED;
+    const dim3 grid((unsigned)(nchunk * s->T));
     const bool batched = pl.KS == 1 && s->K % 4 == 0;      // rows of 4 pairs fetched together (8: no faster)
 #define COMBINE_GO(XT, YH, ST)                                                                          \
     do {                                                                                                \
         if (batched)                                                                                    \
             ODSD_LAUNCH(ODSD_KERNEL_COMBINE, (combine_kernel<XT, YH, ST, 4>), grid, 256, st, y, idx, w, perm, \
                         table, (const XT *)residual, out_f32, (XT *)out_act, row_ss, s->T, s->H, s->K,  \
-                        s->E, pl.KS, P);                                                                \
+                        s->E, pl.KS, P, nchunk);                                                        \
         else                                                                                            \
             ODSD_LAUNCH(ODSD_KERNEL_COMBINE, (combine_kernel<XT, YH, ST, 0>), grid, 256, st, y, idx, w, perm, \
                         table, (const XT *)residual, out_f32, (XT *)out_act, row_ss, s->T, s->H, s->K,  \
-                        s->E, pl.KS, P);                                                                \
+                        s->E, pl.KS, P, nchunk);                                                        \
     } while (0)
 #define COMBINE_Y(XT, ST)                          \
     do {                                           \

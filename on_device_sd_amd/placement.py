@@ -68,24 +68,28 @@ def build_layer_activations(routing_result: RoutingResult, num_experts: int) -> 
                                   routing_scores=scores)
 
 
-def _resident_params(expert_id: ExpertID, expert_cache: Any, parameter_loader: Any):
+def _resident_params(expert_id: ExpertID, expert_cache: Any, parameter_loader: Any, gpu_device: Any):
     """model_runner_utils.py:44-53: shared experts first, then the cache, then the loader's
-    resident copy (``device`` is passed through for loaders that keep several)."""
+    resident copy.  ``gpu_device`` is what the loader's ``get_expert_params`` takes as its
+    ``device`` argument to mean the GPU-resident copy: the reference loader compares it with its
+    own ``DeviceType.GPU`` enum member (parameter_loader.py:613-625), so an engine passes that."""
     if parameter_loader.is_shared_expert(expert_id):
         return parameter_loader.get_shared_expert_params(expert_id)
     if expert_cache.is_cached(expert_id):
         return expert_cache.get(expert_id)
-    return parameter_loader.get_expert_params(expert_id, device="gpu")
+    return parameter_loader.get_expert_params(expert_id, device=gpu_device)
 
 
 def build_prefill_placement(routing_result: RoutingResult, expert_cache: Any,
-                            parameter_loader: Any) -> ExpertPlacement:
+                            parameter_loader: Any, gpu_device: Any = "gpu") -> ExpertPlacement:
     """Placement of a prefill / verify step: every activated expert that is resident goes to
-    ``gpu_expert_params``.  An expert that is not resident is left out (the executor skips it, as
-    the reference skips an expert whose parameters are missing); there is no CPU expert path."""
+    ``gpu_expert_params``.  An expert that is not resident (the lookup gives None) is left out:
+    the executor skips it, as the reference skips an expert whose parameters are missing; there is
+    no CPU expert path.  Pass the loader's own GPU device value as ``gpu_device`` (the reference
+    loader answers any other value with its CPU copy, which the runner refuses)."""
     gpu: Dict[int, Any] = {}
     for expert_id in sorted(routing_result.activated_expert_ids, key=lambda x: x.expert_idx):
-        params = _resident_params(expert_id, expert_cache, parameter_loader)
+        params = _resident_params(expert_id, expert_cache, parameter_loader, gpu_device)
         if params is not None:
             gpu[expert_id.expert_idx] = params
     return ExpertPlacement(gpu_expert_params=gpu, cpu_expert_params={}, routing_result=routing_result)

@@ -77,7 +77,7 @@ class W4MoERunner:
         activated = set(map(ids.__getitem__, self._counts_np.nonzero()[0].tolist()))
         return RoutingResult(layer_idx=layer_idx, topk_indices=idx64, topk_scores=w,
                              activated_expert_ids=activated, dispatch=disp, x_f16=x16,
-                             x_tag=_tensor_tag(flat))
+                             x_tag=_tensor_tag(flat), x_src=hidden_states)
 
     def forward_moe(self, layer_idx: int, attn_output: AttentionOutput,
                     expert_placement: ExpertPlacement) -> torch.Tensor:

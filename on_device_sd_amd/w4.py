@@ -134,12 +134,16 @@ class W4ExpertBank:
         Returns the number of experts loaded."""
         fmt = name_format or self.EXPERT_WEIGHT_NAME
         todo = range(self.num_experts) if experts is None else experts
+        if hasattr(state, "get_tensor"):      # a shard opened with safetensors.safe_open
+            present, fetch = set(state.keys()).__contains__, state.get_tensor
+        else:
+            present, fetch = state.__contains__, state.__getitem__
         loaded = 0
         for e in todo:
             names = [fmt.format(layer=layer_idx, expert=e, proj=p) for p in ("gate", "up", "down")]
-            if not all(n in state for n in names):
+            if not all(present(n) for n in names):
                 continue
-            gate, up, down = (state[n] for n in names)
+            gate, up, down = (fetch(n) for n in names)
             if tuple(gate.shape) != (self.inter, self.hidden) or tuple(up.shape) != (self.inter, self.hidden) \
                     or tuple(down.shape) != (self.hidden, self.inter):
                 raise ValueError(f"layer {layer_idx} expert {e}: unexpected weight shapes "

@@ -42,6 +42,12 @@ def test_argument_checks_need_no_gpu():
     assert lib.odsd_w4_down_splits(C.byref(ok)) >= 1
     bad_h = _lib.MoeShape(8, 200, 8, 2, 256, 1, _lib.DT_BF16, 0)      # H % 128 != 0
     assert lib.odsd_moe_workspace_bytes(C.byref(bad_h)) == 0
+    # shapes whose row offsets do not fit the kernels' 32-bit byte offsets are refused up front
+    huge = _lib.MoeShape(70000, 4096, 8, 8, 4096, 1, _lib.DT_BF16, 0)   # P * I * 2 >= 2^32
+    assert lib.odsd_experts_workspace_bytes(C.byref(huge)) == 0 and lib.odsd_moe_workspace_bytes(C.byref(huge)) == 0
+    assert lib.odsd_w4_gate_up_silu(C.byref(huge), 1 << 20, 1 << 20, 1 << 20, 1 << 20, 1 << 20, 1 << 20, None) == 3
+    long_t = _lib.MoeShape(100000, 1024, 8, 2, 512, 1, _lib.DT_BF16, 0)  # more than 65535 tokens is fine
+    assert lib.odsd_experts_workspace_bytes(C.byref(long_t)) > 0
     big_e = _lib.MoeShape(8, 256, 1024, 2, 256, 1, _lib.DT_BF16, 0)   # E > 512
     assert lib.odsd_router_workspace_bytes(C.byref(big_e)) == 0
     k_gt_e = _lib.MoeShape(8, 256, 4, 8, 256, 1, _lib.DT_BF16, 0)

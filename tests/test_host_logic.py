@@ -83,6 +83,7 @@ def test_prefill_placement_lookup_order_without_gpu():
     from on_device_sd_amd.placement import build_prefill_placement
 
     calls = []
+    GPU = object()                          # stands for the engine's DeviceType.GPU
 
     class Loader:
         def is_shared_expert(self, eid):
@@ -92,6 +93,7 @@ def test_prefill_placement_lookup_order_without_gpu():
             return {"who": "shared"}
         def get_expert_params(self, eid, device=None):
             calls.append(("loader", eid.expert_idx))
+            assert device is GPU            # the engine's own device value reaches the loader
             return None if eid.expert_idx == 5 else {"who": "loader"}
 
     class Cache:
@@ -102,7 +104,7 @@ def test_prefill_placement_lookup_order_without_gpu():
 
     rr = RoutingResult(layer_idx=2, topk_indices=torch.zeros(1, 1, dtype=torch.int64),
                        topk_scores=torch.ones(1, 1), activated_expert_ids={ExpertID(2, e) for e in (3, 4, 5, 6)})
-    pl = build_prefill_placement(rr, Cache(), Loader())
+    pl = build_prefill_placement(rr, Cache(), Loader(), gpu_device=GPU)
     assert {e: p["who"] for e, p in pl.gpu_expert_params.items()} == {3: "shared", 4: "cache", 6: "loader"}
     assert pl.cpu_expert_params == {} and pl.substitution_map == {} and pl.routing_result is rr
     assert ("loader", 3) not in calls and ("loader", 4) not in calls and ("loader", 5) in calls
