@@ -33,6 +33,7 @@
  *   odsd_w4_quantize   quantize_tensor (form, per group)       pre_exp/expert_skip_prediction/quant.py:85-108
  *   odsd_w4_pack       (no counterpart: the reference holds fp16/bf16 weights only;
  *                       parameter_loader.py:424-539 is where a loader would call it)
+ *   odsd_kv_store      store_kvcache                           demo/src/layers/attention.py:32-79
  */
 #ifndef ODSD_MOE_H
 #define ODSD_MOE_H
@@ -198,6 +199,20 @@ int odsd_moe_forward(const odsd_moe_shape *s, const void *x, const void *norm_we
                      int32_t *out_offsets, int32_t *out_perm,
                      const double *row_sumsq_in, double *row_sumsq_out,
                      void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---- KV-cache store (the attention step next to the block) --------------------------------- */
+/* Rows of this step's keys and values to their slots of the paged cache: for i in [0, N)
+ *   row = src_index ? src_index[i] : i;  slot = slot_mapping[i];
+ *   if slot != -1:  k_cache[slot, :] = key[row, :];  v_cache[slot, :] = value[row, :]
+ * key / value: [n_src, D] with row strides key_stride / value_stride (in elements, >= D);
+ * k_cache / v_cache: [num_slots, D] dense; elt_bytes 2 (fp16 / bf16) or 4; bytes are copied as
+ * they are.  Slots must be distinct (two rows with one slot race, as in the reference's kernel);
+ * a slot outside [0, num_slots) or a row outside [0, n_src) is skipped like slot -1.
+ * Stands in for store_kvcache (demo/src/layers/attention.py:32-79) and, with src_index, for the
+ * index_select of the draft tokens in front of it on the verify path (:222-228). */
+int odsd_kv_store(const void *key, const void *value, int64_t key_stride, int64_t value_stride,
+                  void *k_cache, void *v_cache, const int32_t *slot_mapping, const int32_t *src_index,
+                  int32_t N, int32_t n_src, int32_t D, int32_t elt_bytes, int64_t num_slots, void *stream);
 
 /* The same call with every kernel timed, for measurement (no counterpart in the reference):
  * events = 2 * ODSD_N_KERNELS hipEvent_t handles created by the caller; the launch of kernel slot k

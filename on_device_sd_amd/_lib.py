@@ -53,6 +53,8 @@ SIGNATURES = {
     "odsd_moe_workspace_bytes": (C.c_size_t, [_SP]),
     "odsd_moe_forward": (C.c_int, [_SP, _P, _P, C.c_float, _P, _P, C.c_int32, _P, _P, _P, _P, _P, _P,
                                    _P, _P, _P, _P, C.c_size_t, _P]),
+    "odsd_kv_store": (C.c_int, [_P, _P, C.c_int64, C.c_int64, _P, _P, _P, _P, C.c_int32, C.c_int32, C.c_int32,
+                                C.c_int32, C.c_int64, _P]),
     "odsd_moe_forward_events": (C.c_int, [_SP, _P, _P, C.c_float, _P, _P, C.c_int32, _P, _P, _P, _P, _P,
                                           C.c_size_t, _P, _P, _P]),
     "odsd_moe_forward_static": (C.c_int, [_SP, _P, _P, C.c_float, _P, _P, C.c_int32, _P, _P, _P, _P, _P,

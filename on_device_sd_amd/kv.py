@@ -1,0 +1,102 @@
+"""The KV-cache side of a verify step next to the MoE block: where the new keys and values go.
+
+``store_kvcache`` has the arguments and checks of the reference helper of the same name
+(``demo/src/layers/attention.py:57-79``) and runs the gfx950 copy kernel behind ``odsd_kv_store``;
+its optional ``src_index`` folds in the ``index_select`` of the draft tokens that the verify path
+does first (``attention.py:222-228``).  ``SequenceSlots`` and ``build_verify_context`` are the
+host bookkeeping that produces the slot list and the rest of the verify context, with the fields
+and arithmetic of ``SequenceState`` / ``PagedKVCache.get_verify_context``
+(``demo/src/memory/paged_kv_cache.py:127-207, :542-580``); they are plain Python and need no GPU.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence
+
+import torch
+
+from . import _lib
+
+
+def store_kvcache(key: torch.Tensor, value: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                  slot_mapping: torch.Tensor, src_index: Optional[torch.Tensor] = None) -> None:
+    """key, value: [n, num_heads, head_dim]; k_cache, v_cache: [..., D] with D = num_heads*head_dim
+    contiguous rows; slot_mapping: int32 [N] (-1 = no slot).  Without ``src_index`` N == n and row
+    i is stored; with it (int32 [N]) row ``src_index[i]`` is."""
+    if not (key.is_cuda and value.is_cuda and k_cache.is_cuda and v_cache.is_cuda and slot_mapping.is_cuda):
+        raise RuntimeError("the KV store runs on the GPU only (there is no CPU fallback)")
+    n, num_heads, head_dim = key.shape
+    D = num_heads * head_dim
+    assert value.shape == key.shape and key.dtype == value.dtype == k_cache.dtype == v_cache.dtype
+    assert key.stride(-1) == 1 and value.stride(-1) == 1
+    assert key.stride(1) == head_dim and value.stride(1) == head_dim
+    assert k_cache.stride(-1) == 1 and v_cache.stride(-1) == 1
+    assert k_cache.stride(-2) == D and v_cache.stride(-2) == D
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.shape == v_cache.shape
+    N = slot_mapping.numel()
+    if slot_mapping.dtype != torch.int32:
+        slot_mapping = slot_mapping.to(torch.int32)
+    if src_index is None:
+        assert N == n
+    else:
+        assert src_index.numel() == N
+        if src_index.dtype != torch.int32:
+            src_index = src_index.to(torch.int32)
+        src_index = src_index.contiguous()
+    lib = _lib.load()
+    _lib.check(lib.odsd_kv_store(key.data_ptr(), value.data_ptr(), key.stride(0), value.stride(0),
+                                 k_cache.data_ptr(), v_cache.data_ptr(), slot_mapping.contiguous().data_ptr(),
+                                 None if src_index is None else src_index.data_ptr(), N, n, D,
+                                 key.element_size(), k_cache.numel() // D,
+                                 torch.cuda.current_stream().cuda_stream), "odsd_kv_store")
+
+
+@dataclass
+class SequenceSlots:
+    """What the slot arithmetic needs of a sequence (``SequenceState``, paged_kv_cache.py:127-207)."""
+    block_size: int
+    block_table: List[int] = field(default_factory=list)
+    num_tokens: int = 0
+    draft_start_num_tokens: int = 0
+
+    def get_slot_mapping(self, start_pos: int, num_new_tokens: int) -> List[int]:
+        slots = []
+        for i in range(num_new_tokens):
+            pos = start_pos + i
+            block_idx, off = divmod(pos, self.block_size)
+            if block_idx >= len(self.block_table):
+                raise RuntimeError(f"Block index {block_idx} out of range")
+            slots.append(self.block_table[block_idx] * self.block_size + off)
+        return slots
+
+    def get_block_table(self, max_num_blocks: int) -> List[int]:
+        return (self.block_table + [-1] * (max_num_blocks - len(self.block_table)))[:max_num_blocks]
+
+
+def build_verify_context(sequences: Dict[int, SequenceSlots], seq_ids: Sequence[int], device="cuda") -> Dict[str, torch.Tensor]:
+    """``PagedKVCache.get_verify_context`` (paged_kv_cache.py:542-580): per sequence the draft
+    tokens written since ``draft_start_num_tokens`` get their slots; the query holds one more
+    token per sequence (the last accepted one, whose KV is in the cache already), so the rows to
+    store are ``verify_q_indices``."""
+    slot_mapping: List[int] = []
+    context_lens: List[int] = []
+    verify_query_lens: List[int] = []
+    verify_q_indices: List[int] = []
+    max_num_blocks = 0
+    q_offset = 0
+    for seq_id in seq_ids:
+        st = sequences[seq_id]
+        verify_start = st.draft_start_num_tokens
+        num_new = st.num_tokens - verify_start
+        verify_query_lens.append(num_new + 1)
+        if num_new > 0:
+            verify_q_indices.extend(range(q_offset + 1, q_offset + 1 + num_new))
+        q_offset += num_new + 1
+        slot_mapping.extend(st.get_slot_mapping(verify_start, num_new))
+        context_lens.append(st.num_tokens)
+        max_num_blocks = max(max_num_blocks, len(st.block_table))
+    tables = [sequences[s].get_block_table(max_num_blocks) for s in seq_ids]
+    mk = lambda v: torch.tensor(v, dtype=torch.int32, device=device)
+    return {"slot_mapping": mk(slot_mapping), "context_lens": mk(context_lens),
+            "block_tables": mk(tables).reshape(len(seq_ids), max_num_blocks),
+            "verify_query_lens": mk(verify_query_lens), "verify_q_indices": mk(verify_q_indices)}

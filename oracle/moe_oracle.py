@@ -415,3 +415,40 @@ def moe_only_layer(hidden: torch.Tensor, norm_weight: torch.Tensor, gate_weight:
     moe_act = moe.to(hidden.dtype)
     out32 = hidden.to(torch.float32) + moe_act.to(torch.float32)
     return out32.to(hidden.dtype), moe, idx, w
+
+
+# ----------------------------------------------------------------------------
+# KV-cache store and verify context (the attention step next to the block)
+# ----------------------------------------------------------------------------
+def store_kvcache(key: np.ndarray, value: np.ndarray, k_cache: np.ndarray, v_cache: np.ndarray,
+                  slot_mapping, src_index=None) -> None:
+    """demo/src/memory/paged_kv_cache.py:18-45 (the Python statement of the Triton kernel of
+    demo/src/layers/attention.py:32-55): row i of key / value [n, D] goes to row slot_mapping[i]
+    of the caches [slots, D]; slot -1 skips the row.  With src_index the row stored for i is
+    src_index[i]: the verify path's index_select(0, verify_q_indices) in front of the store
+    (attention.py:222-228).  In place."""
+    for i, slot in enumerate(np.asarray(slot_mapping).tolist()):
+        if slot != -1:
+            row = i if src_index is None else int(src_index[i])
+            k_cache[slot] = key[row]
+            v_cache[slot] = value[row]
+
+
+def verify_context(sequences: Sequence[dict], block_size: int):
+    """PagedKVCache.get_verify_context (demo/src/memory/paged_kv_cache.py:542-580) over plain
+    dicts {block_table, num_tokens, draft_start_num_tokens}.  Returns plain lists."""
+    slot_mapping, context_lens, q_lens, q_indices = [], [], [], []
+    q_offset, max_blocks = 0, 0
+    for s in sequences:
+        start = s["draft_start_num_tokens"]
+        new = s["num_tokens"] - start
+        q_lens.append(new + 1)
+        q_indices.extend(range(q_offset + 1, q_offset + 1 + new))
+        q_offset += new + 1
+        for pos in range(start, start + new):
+            slot_mapping.append(s["block_table"][pos // block_size] * block_size + pos % block_size)
+        context_lens.append(s["num_tokens"])
+        max_blocks = max(max_blocks, len(s["block_table"]))
+    tables = [list(s["block_table"]) + [-1] * (max_blocks - len(s["block_table"])) for s in sequences]
+    return {"slot_mapping": slot_mapping, "context_lens": context_lens, "block_tables": tables,
+            "verify_query_lens": q_lens, "verify_q_indices": q_indices}

@@ -78,6 +78,11 @@ def test_argument_checks_need_no_gpu():
     assert lib.odsd_w4_packed_q_bytes(32, 256) == 32 * 256 // 2
     assert lib.odsd_w4_packed_sz_bytes(32, 256) == 32 * 2 * 4
     assert lib.odsd_w4_packed_q_bytes(30, 256) == 0
+    # KV store: argument checks
+    assert lib.odsd_kv_store(None, None, 64, 64, None, None, None, None, 4, 4, 64, 2, 16, None) == 1
+    assert lib.odsd_kv_store(1 << 20, 1 << 20, 32, 64, 1 << 20, 1 << 20, 1 << 20, None, 4, 4, 64, 2, 16, None) == 2
+    assert lib.odsd_kv_store(1 << 20, 1 << 20, 64, 64, 1 << 20, 1 << 20, 1 << 20, None, 4, 4, 64, 3, 16, None) == 7
+    assert lib.odsd_kv_store(None, None, 64, 64, None, None, None, None, 0, 0, 64, 2, 16, None) == 0
     empty = _lib.MoeShape(0, 256, 8, 2, 256, 1, _lib.DT_BF16, 0)       # T == 0 is a no-op
     assert lib.odsd_dispatch(C.byref(empty), 1 << 20, 1 << 20, 1 << 20, 1 << 20, 1 << 20, 1 << 20, None) == 0
 

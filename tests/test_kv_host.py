@@ -1,0 +1,52 @@
+"""Host bookkeeping of the KV side of a verify step (no GPU): slot arithmetic and the verify
+context, against the oracle's restatement and against hand-worked cases."""
+import numpy as np
+import torch
+
+from oracle import moe_oracle as orc
+from on_device_sd_amd.kv import SequenceSlots, build_verify_context
+
+
+def test_slot_mapping_by_hand():
+    s = SequenceSlots(block_size=4, block_table=[7, 2, 9], num_tokens=10)
+    assert s.get_slot_mapping(0, 5) == [28, 29, 30, 31, 8]
+    assert s.get_slot_mapping(6, 4) == [10, 11, 36, 37]
+    assert s.get_block_table(5) == [7, 2, 9, -1, -1]
+    try:
+        s.get_slot_mapping(10, 3)
+    except RuntimeError:
+        pass
+    else:
+        raise AssertionError("positions past the last block must be refused")
+
+
+def test_verify_context_matches_the_oracle_and_a_hand_case():
+    seqs = {
+        5: SequenceSlots(block_size=4, block_table=[3, 0], num_tokens=7, draft_start_num_tokens=4),   # 3 draft tokens
+        9: SequenceSlots(block_size=4, block_table=[1], num_tokens=2, draft_start_num_tokens=2),      # none
+        2: SequenceSlots(block_size=4, block_table=[6, 4, 5], num_tokens=9, draft_start_num_tokens=5),
+    }
+    ctx = build_verify_context(seqs, [5, 9, 2], device="cpu")
+    # by hand: sequence 5 writes positions 4,5,6 -> block 0 offsets 0,1,2; sequence 2 writes 5..8
+    assert ctx["slot_mapping"].tolist() == [0, 1, 2, 17, 18, 19, 20]
+    assert ctx["context_lens"].tolist() == [7, 2, 9]
+    assert ctx["verify_query_lens"].tolist() == [4, 1, 5]
+    assert ctx["verify_q_indices"].tolist() == [1, 2, 3, 6, 7, 8, 9]
+    assert ctx["block_tables"].tolist() == [[3, 0, -1], [1, -1, -1], [6, 4, 5]]
+    assert all(t.dtype == torch.int32 for t in ctx.values())
+    ref = orc.verify_context([dict(block_table=seqs[i].block_table, num_tokens=seqs[i].num_tokens,
+                                   draft_start_num_tokens=seqs[i].draft_start_num_tokens) for i in (5, 9, 2)], 4)
+    for k, v in ref.items():
+        assert ctx[k].tolist() == v, k
+
+
+def test_oracle_store_kvcache_semantics():
+    k = np.arange(12, dtype=np.float32).reshape(4, 3)
+    v = -k
+    kc, vc = np.zeros((6, 3), np.float32), np.zeros((6, 3), np.float32)
+    orc.store_kvcache(k, v, kc, vc, [4, -1, 0, 2])
+    assert kc[4].tolist() == [0, 1, 2] and kc[0].tolist() == [6, 7, 8] and kc[2].tolist() == [9, 10, 11]
+    assert not kc[[1, 3, 5]].any() and np.array_equal(vc, -kc)
+    kc[:] = 0; vc[:] = 0
+    orc.store_kvcache(k, v, kc, vc, [5, 1], src_index=[3, 1])          # the verify path's gather first
+    assert kc[5].tolist() == [9, 10, 11] and kc[1].tolist() == [3, 4, 5] and np.count_nonzero(kc.any(1)) == 2
