@@ -34,6 +34,7 @@
  *   odsd_w4_pack       (no counterpart: the reference holds fp16/bf16 weights only;
  *                       parameter_loader.py:424-539 is where a loader would call it)
  *   odsd_kv_store      store_kvcache                           demo/src/layers/attention.py:32-79
+ *   odsd_paged_attention  _fallback_decode_attention / flash_attn_with_kvcache   attention.py:252-352
  */
 #ifndef ODSD_MOE_H
 #define ODSD_MOE_H
@@ -60,7 +61,7 @@ typedef enum odsd_status {
                                  ODSD_STATIC_SCRATCH_BYTES of scratch memory             */
 } odsd_status;
 
-enum { ODSD_DT_F32 = 0, ODSD_DT_BF16 = 1 };
+enum { ODSD_DT_F32 = 0, ODSD_DT_BF16 = 1, ODSD_DT_F16 = 2 /* attention entry point only */ };
 
 /* Shape of one MoE layer call.  Rules: H % 128 == 0, I % 128 == 0, 1 <= K <= E <= 512,
  * K <= 64, T >= 0 (T == 0 is a no-op). */
@@ -213,6 +214,26 @@ int odsd_moe_forward(const odsd_moe_shape *s, const void *x, const void *norm_we
 int odsd_kv_store(const void *key, const void *value, int64_t key_stride, int64_t value_stride,
                   void *k_cache, void *v_cache, const int32_t *slot_mapping, const int32_t *src_index,
                   int32_t N, int32_t n_src, int32_t D, int32_t elt_bytes, int64_t num_slots, void *stream);
+
+/* Causal attention of a decode / verify step over the paged KV cache.
+ *   q            [n_tokens, num_heads, head_dim]: the sequences' query tokens one after the other,
+ *                q_lens[s] of them for sequence s (q_lens == NULL: one each, a decode step)
+ *   k_cache, v_cache  [num_slots, num_kv_heads * head_dim]; position p of sequence s lives in slot
+ *                block_tables[s][p / block_size] * block_size + p % block_size
+ *   context_lens [n_seqs]: cached tokens of the sequence INCLUDING this step's (stored before)
+ *   query j of sequence s attends positions 0 .. context_lens[s] - q_lens[s] + j; query head h
+ *   reads KV head h / (num_heads / num_kv_heads); scores scaled by softmax_scale; fp32 softmax
+ *   out          [n_tokens, num_heads, head_dim] in the dtype of q (ODSD_DT_BF16 or ODSD_DT_F16)
+ * max_q_len: an upper bound of q_lens (sizes the launch); head_dim 64 or 128.
+ * Stands in for Qwen3Attention._fallback_decode_attention and the flash_attn_with_kvcache call
+ * it replaces (demo/src/layers/attention.py:252-352), on the context of
+ * PagedKVCache.get_verify_context / get_attention_context (demo/src/memory/paged_kv_cache.py:500-580). */
+int odsd_paged_attention(const void *q, const void *k_cache, const void *v_cache,
+                         const int32_t *block_tables, const int32_t *context_lens,
+                         const int32_t *q_lens, int32_t n_seqs, int32_t max_q_len,
+                         int32_t num_heads, int32_t num_kv_heads, int32_t head_dim,
+                         int32_t block_size, int32_t max_blocks, int64_t num_slots,
+                         float softmax_scale, int32_t dtype, void *out, void *stream);
 
 /* The same call with every kernel timed, for measurement (no counterpart in the reference):
  * events = 2 * ODSD_N_KERNELS hipEvent_t handles created by the caller; the launch of kernel slot k

@@ -15,6 +15,7 @@ LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), LIB_NAME)
 
 DT_F32 = 0
 DT_BF16 = 1
+DT_F16 = 2
 TABLE_COLS = 4
 
 
@@ -55,6 +56,8 @@ SIGNATURES = {
                                    _P, _P, _P, _P, C.c_size_t, _P]),
     "odsd_kv_store": (C.c_int, [_P, _P, C.c_int64, C.c_int64, _P, _P, _P, _P, C.c_int32, C.c_int32, C.c_int32,
                                 C.c_int32, C.c_int64, _P]),
+    "odsd_paged_attention": (C.c_int, [_P, _P, _P, _P, _P, _P, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
+                                       C.c_int32, C.c_int32, C.c_int64, C.c_float, C.c_int32, _P, _P]),
     "odsd_moe_forward_events": (C.c_int, [_SP, _P, _P, C.c_float, _P, _P, C.c_int32, _P, _P, _P, _P, _P,
                                           C.c_size_t, _P, _P, _P]),
     "odsd_moe_forward_static": (C.c_int, [_SP, _P, _P, C.c_float, _P, _P, C.c_int32, _P, _P, _P, _P, _P,

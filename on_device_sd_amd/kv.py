@@ -51,6 +51,45 @@ def store_kvcache(key: torch.Tensor, value: torch.Tensor, k_cache: torch.Tensor,
                                  torch.cuda.current_stream().cuda_stream), "odsd_kv_store")
 
 
+def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, context: Dict[str, torch.Tensor],
+                    num_kv_heads: int, block_size: int, softmax_scale: Optional[float] = None,
+                    max_q_len: Optional[int] = None) -> torch.Tensor:
+    """Causal attention of a decode / verify step over the paged cache: what
+    ``Qwen3Attention.forward`` computes after the KV store (``demo/src/layers/attention.py:252-352``).
+    q: [n_tokens, num_heads, head_dim] (bf16 / fp16); k_cache, v_cache: [..., num_kv_heads*head_dim]
+    holding this step's keys and values already; ``context``: ``block_tables`` int32
+    [n_seqs, max_blocks], ``context_lens`` int32 [n_seqs] and, for a verify step,
+    ``verify_query_lens`` int32 [n_seqs] (absent: one query token per sequence).  Returns
+    [n_tokens, num_heads, head_dim] in the dtype of q.  ``max_q_len`` bounds the query lengths
+    (default: n_tokens, which is always safe)."""
+    if not (q.is_cuda and k_cache.is_cuda and v_cache.is_cuda):
+        raise RuntimeError("paged attention runs on the GPU only (there is no CPU fallback)")
+    n_tokens, num_heads, head_dim = q.shape
+    D = num_kv_heads * head_dim
+    assert q.is_contiguous() and k_cache.is_contiguous() and v_cache.is_contiguous()
+    assert k_cache.shape[-1] == D and v_cache.shape == k_cache.shape and q.dtype == k_cache.dtype == v_cache.dtype
+    dt = {torch.bfloat16: _lib.DT_BF16, torch.float16: _lib.DT_F16}.get(q.dtype)
+    if dt is None:
+        raise TypeError("paged attention takes bfloat16 or float16")
+    tables = context["block_tables"].to(torch.int32).contiguous()
+    lens = context["context_lens"].to(torch.int32).contiguous()
+    q_lens = context.get("verify_query_lens")
+    if q_lens is not None:
+        q_lens = q_lens.to(torch.int32).contiguous()
+    n_seqs = lens.numel()
+    out = torch.empty_like(q)
+    if n_seqs == 0 or n_tokens == 0:
+        return out
+    scale = head_dim ** -0.5 if softmax_scale is None else softmax_scale
+    lib = _lib.load()
+    _lib.check(lib.odsd_paged_attention(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), tables.data_ptr(),
+                                        lens.data_ptr(), None if q_lens is None else q_lens.data_ptr(), n_seqs,
+                                        max_q_len or n_tokens, num_heads, num_kv_heads, head_dim, block_size,
+                                        tables.shape[1], k_cache.numel() // D, scale, dt, out.data_ptr(),
+                                        torch.cuda.current_stream().cuda_stream), "odsd_paged_attention")
+    return out
+
+
 @dataclass
 class SequenceSlots:
     """What the slot arithmetic needs of a sequence (``SequenceState``, paged_kv_cache.py:127-207)."""

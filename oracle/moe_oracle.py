@@ -452,3 +452,33 @@ def verify_context(sequences: Sequence[dict], block_size: int):
     tables = [list(s["block_table"]) + [-1] * (max_blocks - len(s["block_table"])) for s in sequences]
     return {"slot_mapping": slot_mapping, "context_lens": context_lens, "block_tables": tables,
             "verify_query_lens": q_lens, "verify_q_indices": q_indices}
+
+
+def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables,
+                    context_lens, q_lens, num_kv_heads: int, block_size: int, scale: float) -> torch.Tensor:
+    """Qwen3Attention._fallback_decode_attention (demo/src/layers/attention.py:290-352) in fp32:
+    per sequence the cached K / V rows of positions 0 .. context_len-1 are gathered by slot
+    (block_table[p // block_size] * block_size + p % block_size), repeated over the query heads of
+    their group (repeat_interleave), and F.scaled_dot_product_attention runs with the additive
+    mask that forbids key > query + (k_len - q_len).  q: [n_tokens, H, HD]; caches
+    [slots, KVH*HD]; q_lens None = one query token per sequence."""
+    n_tokens, H, HD = q.shape
+    kc = k_cache.reshape(-1, num_kv_heads * HD).to(torch.float32)
+    vc = v_cache.reshape(-1, num_kv_heads * HD).to(torch.float32)
+    qf = q.to(torch.float32)
+    outs, q0 = [], 0
+    for i, L in enumerate(np.asarray(context_lens).tolist()):
+        ql = 1 if q_lens is None else int(np.asarray(q_lens)[i])
+        q_seq = qf[q0:q0 + ql]
+        q0 += ql
+        table = np.asarray(block_tables[i]).tolist()
+        slots = torch.tensor([table[p // block_size] * block_size + p % block_size for p in range(L)], dtype=torch.long)
+        k_seq = kc.index_select(0, slots).view(L, num_kv_heads, HD).repeat_interleave(H // num_kv_heads, dim=1)
+        v_seq = vc.index_select(0, slots).view(L, num_kv_heads, HD).repeat_interleave(H // num_kv_heads, dim=1)
+        disallow = torch.triu(torch.ones((ql, L), dtype=torch.bool), diagonal=L - ql + 1)
+        bias = torch.zeros((ql, L)).masked_fill(disallow, float("-inf"))
+        o = F.scaled_dot_product_attention(q_seq.transpose(0, 1).unsqueeze(0), k_seq.transpose(0, 1).unsqueeze(0),
+                                           v_seq.transpose(0, 1).unsqueeze(0), attn_mask=bias, dropout_p=0.0,
+                                           is_causal=False, scale=scale)
+        outs.append(o.squeeze(0).transpose(0, 1))
+    return torch.cat(outs, dim=0)

@@ -63,3 +63,51 @@ def test_verify_step_store_with_gather_and_strided_rows(dev):
     sel = ctx["verify_q_indices"].to(torch.long)
     odsd.store_kvcache(k.index_select(0, sel), v.index_select(0, sel), cache2[0], cache2[1], ctx["slot_mapping"])
     assert torch.equal(cache, cache2)
+
+
+ATTN_CASES = [
+    # dtype, H, KVH, HD, block_size, (context_len, q_len) per sequence (q_len None column -> decode step)
+    (torch.bfloat16, 32, 4, 128, 16, [(600, 8), (37, 1), (129, 5), (8, 8), (1000, 3)]),   # Qwen3-30B-A3B heads, verify step
+    (torch.bfloat16, 32, 4, 128, 256, [(700, 8), (300, 8)]),                              # the reference's block size
+    (torch.float16, 8, 8, 64, 8, [(95, 4), (1, 1), (33, 2)]),                             # no grouping, head_dim 64
+    (torch.bfloat16, 16, 2, 128, 16, [(260, 12), (64, 9)]),                               # 96 and 72 query rows: two row groups
+    (torch.float16, 32, 4, 128, 32, [(513, None), (40, None), (1, None), (250, None)]),   # decode step
+]
+
+
+@pytest.mark.parametrize("dtype,H,KVH,HD,bs,seqs", ATTN_CASES)
+def test_paged_attention_vs_oracle(dev, dtype, H, KVH, HD, bs, seqs):
+    print("paged attention", dtype, H, KVH, HD, bs, seqs, flush=True)
+    import on_device_sd_amd as odsd
+    g = torch.Generator().manual_seed(H + HD + bs)
+    decode = seqs[0][1] is None
+    n_blocks_per = [-(-L // bs) for L, _ in seqs]
+    total_blocks = sum(n_blocks_per) + 3
+    perm = torch.randperm(total_blocks, generator=g).tolist()
+    tables, at = [], 0
+    for nb in n_blocks_per:
+        tables.append(perm[at:at + nb]); at += nb
+    max_blocks = max(n_blocks_per)
+    bt = torch.tensor([t + [-1] * (max_blocks - len(t)) for t in tables], dtype=torch.int32)
+    D = KVH * HD
+    kc = torch.randn(total_blocks * bs, D, generator=g).to(dtype)
+    vc = torch.randn(total_blocks * bs, D, generator=g).to(dtype)
+    lens = torch.tensor([L for L, _ in seqs], dtype=torch.int32)
+    qlens = None if decode else torch.tensor([ql for _, ql in seqs], dtype=torch.int32)
+    n_tok = len(seqs) if decode else int(qlens.sum())
+    q = torch.randn(n_tok, H, HD, generator=g).to(dtype)
+    ctx = {"block_tables": bt.to(dev), "context_lens": lens.to(dev)}
+    if not decode:
+        ctx["verify_query_lens"] = qlens.to(dev)
+    out = odsd.paged_attention(q.to(dev), kc.to(dev), vc.to(dev), ctx, KVH, bs,
+                               max_q_len=None if decode else int(qlens.max()))
+    torch.cuda.synchronize()
+    ref = orc.paged_attention(q, kc, vc, bt.numpy(), lens.numpy(), None if decode else qlens.numpy(), KVH, bs, HD ** -0.5)
+    err = (out.float().cpu() - ref).abs().max().item()
+    tol = 2e-2 if dtype == torch.bfloat16 else 3e-3       # output rounding + P in the storage dtype
+    print(f"  max-abs error {err:.3e} (max|ref| {ref.abs().max().item():.2f})", flush=True)
+    assert err <= tol
+    # a second run gives the same bits
+    out2 = odsd.paged_attention(q.to(dev), kc.to(dev), vc.to(dev), ctx, KVH, bs,
+                                max_q_len=None if decode else int(qlens.max()))
+    assert torch.equal(out, out2)

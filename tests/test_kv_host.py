@@ -50,3 +50,33 @@ def test_oracle_store_kvcache_semantics():
     kc[:] = 0; vc[:] = 0
     orc.store_kvcache(k, v, kc, vc, [5, 1], src_index=[3, 1])          # the verify path's gather first
     assert kc[5].tolist() == [9, 10, 11] and kc[1].tolist() == [3, 4, 5] and np.count_nonzero(kc.any(1)) == 2
+
+
+def test_oracle_paged_attention_against_plain_softmax():
+    """The oracle's attention (library SDPA over gathered rows) against a scalar restatement of
+    softmax(q k^T * scale + causal mask) v on a tiny case, and its decode special case."""
+    g = torch.Generator().manual_seed(0)
+    H, KVH, HD, bs = 4, 2, 8, 4
+    kc = torch.randn(5 * bs, KVH * HD, generator=g)
+    vc = torch.randn(5 * bs, KVH * HD, generator=g)
+    tables = [[3, 1, -1], [0, 2, 4]]
+    lens, qlens = [6, 11], [3, 2]
+    q = torch.randn(5, H, HD, generator=g)
+    out = orc.paged_attention(q, kc, vc, tables, lens, qlens, KVH, bs, 0.3)
+    q0 = 0
+    for s in range(2):
+        L, ql = lens[s], qlens[s]
+        slot = lambda p: tables[s][p // bs] * bs + p % bs
+        for j in range(ql):
+            for h in range(H):
+                kvh = h // (H // KVH)
+                last = L - ql + j
+                sc = [float(q[q0 + j, h] @ kc[slot(p), kvh * HD:(kvh + 1) * HD]) * 0.3 for p in range(last + 1)]
+                m = max(sc)
+                w = [np.exp(x - m) for x in sc]
+                ref = sum(wi * vc[slot(p), kvh * HD:(kvh + 1) * HD] for p, wi in enumerate(w)) / sum(w)
+                assert torch.allclose(out[q0 + j, h], ref.to(torch.float32), atol=1e-5)
+        q0 += ql
+    dec = orc.paged_attention(q[:2], kc, vc, tables, lens, None, KVH, bs, 0.3)
+    one = orc.paged_attention(q[:2], kc, vc, tables, lens, [1, 1], KVH, bs, 0.3)
+    assert torch.equal(dec, one)
