@@ -225,6 +225,8 @@ int odsd_kv_store(const void *key, const void *value, int64_t key_stride, int64_
  *   reads KV head h / (num_heads / num_kv_heads); scores scaled by softmax_scale; fp32 softmax
  *   out          [n_tokens, num_heads, head_dim] in the dtype of q (ODSD_DT_BF16 or ODSD_DT_F16)
  * max_q_len: an upper bound of q_lens (sizes the launch); head_dim 64 or 128.
+ * workspace: odsd_paged_attention_workspace_bytes(...) bytes (with few sequences the keys of one
+ * sequence are shared out between workgroups, whose partial results land there).
  * Stands in for Qwen3Attention._fallback_decode_attention and the flash_attn_with_kvcache call
  * it replaces (demo/src/layers/attention.py:252-352), on the context of
  * PagedKVCache.get_verify_context / get_attention_context (demo/src/memory/paged_kv_cache.py:500-580). */
@@ -233,7 +235,11 @@ int odsd_paged_attention(const void *q, const void *k_cache, const void *v_cache
                          const int32_t *q_lens, int32_t n_seqs, int32_t max_q_len,
                          int32_t num_heads, int32_t num_kv_heads, int32_t head_dim,
                          int32_t block_size, int32_t max_blocks, int64_t num_slots,
-                         float softmax_scale, int32_t dtype, void *out, void *stream);
+                         float softmax_scale, int32_t dtype, void *out, void *workspace,
+                         size_t workspace_bytes, void *stream);
+size_t odsd_paged_attention_workspace_bytes(int32_t n_seqs, int32_t max_q_len, int32_t num_heads,
+                                            int32_t num_kv_heads, int32_t head_dim, int32_t block_size,
+                                            int32_t max_blocks);
 
 /* The same call with every kernel timed, for measurement (no counterpart in the reference):
  * events = 2 * ODSD_N_KERNELS hipEvent_t handles created by the caller; the launch of kernel slot k

@@ -1,6 +1,6 @@
 // Causal attention of a decode / verify step over the paged KV cache (gfx950).
 //
-// One workgroup per (sequence, KV head, group of 64 query rows); a query row is one (token, query
+// One workgroup per (sequence, KV head, group of 64 query rows, slice of the keys); a query row is one (token, query
 // head) pair of the KV head's group, so with grouped-query attention a verify step of 8 tokens and
 // 8 query heads per KV head fills the 64 rows.  Each of the 4 wavefronts owns 16 rows and walks
 // the sequence's cached keys 32 at a time:
@@ -11,6 +11,10 @@
 //   * online softmax in fp32 (running maximum and sum per row, exp2 with the scale folded in);
 //   * O += P V with V^T as the B operand: the 32 x head_dim tile of V is transposed through LDS
 //     once per workgroup (double buffered, one barrier per tile) and shared by the wavefronts.
+// A verify step has few (sequence, KV head) pairs and long key lists, so the keys of one sequence
+// are cut into `splits` slices handled by different workgroups; each leaves its running maximum,
+// sum and unnormalised output, and a small second kernel merges the slices of a row (the usual
+// rescaling by exp2(m_slice - m_all)), in slice order.
 // The cache is addressed through the sequence's block table exactly as the reference gathers it:
 // position p lives in slot block_table[p / block_size] * block_size + p % block_size.
 //
@@ -18,6 +22,7 @@
 // of the cached K/V by slot, repeat_interleave for GQA, causal mask with offset k_len - q_len,
 // scaled_dot_product_attention) and the flash_attn_with_kvcache call it stands in for (:252-272).
 #include "common.h"
+#include <type_traits>
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 
@@ -32,6 +37,8 @@ struct AttnParams {
     int n_seqs, H, KVH, max_blocks, block_size;
     int64_t num_slots;
     float scale_log2e;         // softmax scale * log2(e)
+    int splits;                // workgroups sharing one sequence's keys (blockIdx.z)
+    float *part;               // splits > 1: partial results [seq, kvh, row group][split][64][HD + 2]
 };
 
 template <typename T> struct AttnT;
@@ -54,8 +61,17 @@ template <> struct AttnT<__bf16> {
 // lane group kq feeds to one product step (4 of each 16-key half) sit next to each other
 __device__ __forceinline__ int vt_pos(int key) { return 8 * ((key & 15) >> 2) + 4 * (key >> 4) + (key & 3); }
 
-template <typename T, int HD>
-__global__ __launch_bounds__(256) void paged_attn_kernel(const AttnParams p) {
+// first query token of sequence seq: the sum of the query lengths before it, one wavefront-wide pass
+__device__ __forceinline__ int attn_first_token(const int32_t *q_lens, int seq) {
+    int part = 0;
+    for (int i = threadIdx.x & 63; i < seq; i += 64) part += q_lens[i];
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) part += __shfl_xor(part, d, ODSD_WAVE);
+    return part;
+}
+
+template <typename T, int HD, bool ALIGNED>
+__global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) {
     typedef typename AttnT<T>::V8 V8;
     constexpr int NJ = HD / 32;          // 32-dim steps of the score product
     constexpr int NDB = HD / 16;         // 16-dim column blocks of the output
@@ -68,12 +84,10 @@ __global__ __launch_bounds__(256) void paged_attn_kernel(const AttnParams p) {
     const int c = lane & 15, kq = lane >> 4;
     const int Gq = p.H / p.KVH;
     const int L = p.context_lens[seq];
-    int ql = 1, q0 = 0;
+    int ql = 1, q0 = seq;
     if (p.q_lens) {
         ql = p.q_lens[seq];
-        for (int i = 0; i < seq; ++i) q0 += p.q_lens[i];
-    } else {
-        q0 = seq;
+        q0 = attn_first_token(p.q_lens, seq);
     }
     const int rows_total = ql * Gq;
     if (L <= 0 || ql <= 0 || (int)blockIdx.y * 64 >= rows_total) return;
@@ -82,15 +96,6 @@ __global__ __launch_bounds__(256) void paged_attn_kernel(const AttnParams p) {
     const int D = p.KVH * HD;
     const uint16_t *kc = (const uint16_t *)p.k_cache, *vc = (const uint16_t *)p.v_cache;
     const int32_t *bt = p.block_tables + (size_t)seq * p.max_blocks;
-
-    // slot of position pos (clamped into the sequence; a broken table entry reads slot 0, masked below)
-    auto slot_of = [&](int pos) -> int64_t {
-        const int pc = min(pos, L - 1);
-        const int blk = pc / p.block_size;
-        const int64_t b = blk < p.max_blocks ? bt[blk] : -1;
-        const int64_t s = b * p.block_size + (pc - blk * p.block_size);
-        return (s >= 0 && s < p.num_slots) ? s : 0;
-    };
 
     // this lane's query row (B operand of S^T = K Q^T: lane (c, kq) holds Q[row c][32 j + 8 kq ..])
     const int row = row0 + c;
@@ -113,73 +118,132 @@ __global__ __launch_bounds__(256) void paged_attn_kernel(const AttnParams p) {
 #pragma unroll
     for (int db = 0; db < NDB; ++db) o[db] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    // Software pipeline over the 32-key tiles: the cache slots of a tile are looked up two tiles
-    // ahead (block table -> slot is a dependent load), its K fragments and V pieces are fetched one
-    // tile ahead, so that a tile's products never wait for a chain of two loads.
+    // Software pipeline over the 32-key tiles, two tiles deep: during tile `it` the K fragments and
+    // V pieces of tile it + 2 are fetched into the register set tile `it` has just finished with,
+    // V of tile it + 1 goes transposed into the other LDS buffer, and the block-table entries of
+    // tile it + 3 are requested BEFORE the fetches (the load counter retires in order: a younger
+    // table read awaited by the next tile would otherwise drain the big fetches issued before it).
+    // The steady-state tiles fetch unconditionally and the last two tiles are compiled without the
+    // fetch, so that no wait is placed after a join of "fetched" and "did not fetch".
     //   K: lane (c, kq) reads 16 bytes of key row 16 t + c for each 32-dim step (the A operand)
     //   V: piece = tid + 256 u -> key = piece / (HD / 8), dims 8 * (piece % (HD / 8)) ..
-    int64_t kslot[2], vslot[PIECES];
-    auto lookup = [&](int k0) {
+    // ALIGNED (block_size a multiple of 32): a tile lies in one cache block, so its table entry is
+    // one wavefront-uniform read; otherwise every lane reads the entry of its own key.
+    constexpr int NE = ALIGNED ? 1 : 2 + PIECES;        // table entries a tile needs per lane
+    const int k_last = L - 1;
+    const int bs = p.block_size;
+    auto entry_at = [&](int pos) -> int32_t { return bt[min(min(pos, k_last) / bs, p.max_blocks - 1)]; };
+    auto request = [&](int k0, int32_t (&e)[NE]) {
+        if constexpr (ALIGNED) {
+            e[0] = entry_at(k0);
+        } else {
 #pragma unroll
-        for (int t = 0; t < 2; ++t) kslot[t] = slot_of(k0 + 16 * t + c);
+            for (int t = 0; t < 2; ++t) e[t] = entry_at(k0 + 16 * t + c);
 #pragma unroll
-        for (int u = 0; u < PIECES; ++u) vslot[u] = slot_of(k0 + (tid + 256 * u) / (HD / 8));
-    };
-    uint4_t kreg[2][NJ], vreg[PIECES];
-    auto fetch = [&]() {
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            const uint16_t *kp = kc + kslot[t] * D + kvh * HD + 8 * kq;
-#pragma unroll
-            for (int j = 0; j < NJ; ++j) kreg[t][j] = *(const uint4_t *)(kp + 32 * j);
-        }
-#pragma unroll
-        for (int u = 0; u < PIECES; ++u) {
-            const int ch = (tid + 256 * u) % (HD / 8);
-            vreg[u] = *(const uint4_t *)(vc + vslot[u] * D + kvh * HD + 8 * ch);
+            for (int u = 0; u < PIECES; ++u) e[2 + u] = entry_at(k0 + (tid + 256 * u) / (HD / 8));
         }
     };
-    auto store_v = [&](int buf) {
+    // slot of position pos (clamped into the sequence) in the block whose table entry is b; an
+    // entry that is negative, beyond the table or beyond the cache reads slot 0
+    auto slot_in = [&](int32_t b, int pos) -> int64_t {
+        const int pc = min(pos, k_last);
+        const int blk = pc / bs;
+        const int64_t sl = (int64_t)b * bs + (pc - blk * bs);
+        return (b >= 0 && blk < p.max_blocks && sl < p.num_slots) ? sl : 0;
+    };
+    uint4_t kreg[2][2][NJ], vreg[2][PIECES];
+    // fetch of the tile at k0, whose table entries are e
+    auto fetch = [&](auto set, int k0, const int32_t (&e)[NE]) {
+        constexpr int S = decltype(set)::value;
+        if constexpr (ALIGNED) {
+            // everything about the block is wavefront-uniform: one 64-bit base per tile, and a lane
+            // adds the 32-bit offset of its row (clamped to the sequence's last key in the tile)
+            const int k0c = min(k0, k_last & ~31);
+            const int blk = k0c / bs;
+            const int32_t b = e[0];
+            const bool ok = b >= 0 && blk < p.max_blocks && ((int64_t)b + 1) * bs <= p.num_slots;
+            const int64_t slot0 = ok ? (int64_t)b * bs + (k0c - blk * bs) : 0;
+            const int lim = ok ? k_last - k0c : 0;
+            const size_t base = (size_t)slot0 * D + kvh * HD;
+            const uint16_t *kb = kc + base, *vb = vc + base;
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const uint32_t off = (uint32_t)min(16 * t + c, lim) * (uint32_t)D + 8 * kq;
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) kreg[S][t][j] = *(const uint4_t *)(kb + off + 32 * j);
+            }
+#pragma unroll
+            for (int u = 0; u < PIECES; ++u) {
+                const int piece = tid + 256 * u;
+                const uint32_t off = (uint32_t)min(piece / (HD / 8), lim) * (uint32_t)D + 8 * (piece % (HD / 8));
+                vreg[S][u] = *(const uint4_t *)(vb + off);
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const int64_t sl = slot_in(e[t], k0 + 16 * t + c);
+                const uint16_t *kp = kc + sl * D + kvh * HD + 8 * kq;
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) kreg[S][t][j] = *(const uint4_t *)(kp + 32 * j);
+            }
+#pragma unroll
+            for (int u = 0; u < PIECES; ++u) {
+                const int piece = tid + 256 * u;
+                const int64_t sl = slot_in(e[2 + u], k0 + piece / (HD / 8));
+                vreg[S][u] = *(const uint4_t *)(vc + sl * D + kvh * HD + 8 * (piece % (HD / 8)));
+            }
+        }
+    };
+    // V^T tile in LDS: row = dim, 32 key positions (+ pad); the 8-position segment index is XORed
+    // with (dim / 8) & 3 so that the 16 lanes writing one key's 16 dim chunks spread over the banks
+    auto store_v = [&](auto set, int buf) {
+        constexpr int S = decltype(set)::value;
 #pragma unroll
         for (int u = 0; u < PIECES; ++u) {
             const int piece = tid + 256 * u;
             const int key = piece / (HD / 8), ch = piece % (HD / 8);
-            const int pos = vt_pos(key);
-            const uint32_t w[4] = {vreg[u].x, vreg[u].y, vreg[u].z, vreg[u].w};
+            const int pos = vt_pos(key) ^ (8 * (ch & 3));
+            const uint32_t w[4] = {vreg[S][u].x, vreg[S][u].y, vreg[S][u].z, vreg[S][u].w};
 #pragma unroll
             for (int i = 0; i < 8; ++i)
                 vt[buf][(8 * ch + i) * VT_LD + pos] = (uint16_t)(w[i >> 1] >> (16 * (i & 1)));
         }
     };
 
-    const int n_tiles = (L + 31) / 32;
-    lookup(0);
-    fetch();                                            // tile 0
-    lookup(32);                                         // slots of tile 1 (clamped past the end)
-    store_v(0);
-    V8 kf[2][NJ];
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int j = 0; j < NJ; ++j) kf[t][j] = __builtin_bit_cast(V8, kreg[t][j]);
-    __syncthreads();
-    for (int it = 0; it < n_tiles; ++it) {
-        const int k0 = it * 32, buf = it & 1;
-        const bool more = it + 1 < n_tiles;
-        if (more) {
-            fetch();                                    // tile it + 1, in flight while this one is computed
-            lookup(k0 + 64);                            // slots of tile it + 2
-        }
+    // this workgroup's slice of the 32-key tiles
+    const int all_tiles = (L + 31) / 32;
+    const int per_split = (all_tiles + p.splits - 1) / p.splits;
+    const int t_begin = min(all_tiles, (int)blockIdx.z * per_split);
+    const int n_tiles = min(all_tiles, t_begin + per_split) - t_begin;
+    const int kbase = t_begin * 32;
+    int32_t pend[NE];                                   // entries of the tile after the newest fetched one
+
+    // one tile; S: the register set holding its K. FETCH: tile it + 2 exists and is fetched (and
+    // the entries of tile it + 3 requested); STORE: tile it + 1 exists and its V goes to LDS
+    auto tile = [&](auto set, auto fetch_c, auto store_c, int it) {
+        constexpr int S = decltype(set)::value;
+        constexpr bool FETCH = decltype(fetch_c)::value, STORE = decltype(store_c)::value;
+        const int k0 = kbase + it * 32, buf = it & 1;
+        float4_t st[2];
         if (wave_active) {
             // scores S^T[key][row] for the two 16-key halves
-            float4_t st[2];
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
                 float4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int j = 0; j < NJ; ++j) acc = AttnT<T>::mfma(kf[t][j], qf[j], acc);
+                for (int j = 0; j < NJ; ++j)
+                    acc = AttnT<T>::mfma(__builtin_bit_cast(V8, kreg[S][t][j]), qf[j], acc);
                 st[t] = acc;
             }
+        }
+        if constexpr (FETCH) {
+            int32_t now[NE];
+#pragma unroll
+            for (int i = 0; i < NE; ++i) now[i] = pend[i];
+            request(k0 + 96, pend);
+            fetch(set, k0 + 64, now);
+        }
+        if (wave_active) {
             // lane (c, kq) holds keys k0 + 16 t + 4 kq + i of query row c: mask, running max and sum
             float sv[8];
             float mx = -INFINITY;
@@ -199,12 +263,12 @@ __global__ __launch_bounds__(256) void paged_attn_kernel(const AttnParams p) {
             const float m_new = fmaxf(m_run, mx);
             // a row with nothing to attend yet keeps m = -inf: use 0 as the reference point then
             const float m_ref = m_new == -INFINITY ? 0.0f : m_new;
-            const float alpha = exp2f(m_run - m_ref);        // m_run = -inf -> 0
+            const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);        // m_run = -inf -> 0
             float ps = 0.0f;
             uint16_t pb[8];
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const float e = exp2f(sv[i] - m_ref);         // masked -> 0
+                const float e = __builtin_amdgcn_exp2f(sv[i] - m_ref);         // masked -> 0
                 pb[i] = AttnT<T>::from_f32(e);
                 ps += e;
             }
@@ -220,24 +284,76 @@ __global__ __launch_bounds__(256) void paged_attn_kernel(const AttnParams p) {
             float al[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) al[i] = __shfl(alpha, 4 * kq + i, ODSD_WAVE);
+            // once the running maxima have settled no row of the wavefront rescales any more
+            if (__any(alpha != 1.0f)) {
+#pragma unroll
+                for (int db = 0; db < NDB; ++db) {
+                    o[db].x *= al[0]; o[db].y *= al[1]; o[db].z *= al[2]; o[db].w *= al[3];
+                }
+            }
 #pragma unroll
             for (int db = 0; db < NDB; ++db) {
-                const V8 vf = __builtin_bit_cast(V8, *(const uint4_t *)&vt[buf][(16 * db + c) * VT_LD + 8 * kq]);
-                float4_t acc = o[db];
-                acc.x *= al[0]; acc.y *= al[1]; acc.z *= al[2]; acc.w *= al[3];
-                o[db] = AttnT<T>::mfma(pf, vf, acc);
+                const int seg = kq ^ ((2 * db + (c >> 3)) & 3);
+                const V8 vf = __builtin_bit_cast(V8, *(const uint4_t *)&vt[buf][(16 * db + c) * VT_LD + 8 * seg]);
+                o[db] = AttnT<T>::mfma(pf, vf, o[db]);
             }
         }
-        if (more) {
-            store_v(buf ^ 1);
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-#pragma unroll
-                for (int j = 0; j < NJ; ++j) kf[t][j] = __builtin_bit_cast(V8, kreg[t][j]);
-        }
+        // V of tile it + 1 (other set, fetched during tile it - 1) into the other LDS buffer
+        if constexpr (STORE) store_v(std::integral_constant<int, S ^ 1>{}, buf ^ 1);
         __syncthreads();
+    };
+
+    if (n_tiles > 0) {
+        const std::integral_constant<int, 0> s0;
+        const std::integral_constant<int, 1> s1;
+        const std::true_type yes;
+        const std::false_type no;
+        // prologue: tiles 0 and 1 fetched, V of tile 0 in LDS, the entries of tile 2 requested
+        request(kbase, pend);
+        fetch(s0, kbase, pend);
+        if (n_tiles > 1) {
+            request(kbase + 32, pend);
+            fetch(s1, kbase + 32, pend);
+        }
+        request(kbase + 64, pend);
+        store_v(s0, 0);
+        __syncthreads();
+        int it = 0;
+        for (; it + 3 < n_tiles; it += 2) {
+            tile(s0, yes, yes, it);
+            tile(s1, yes, yes, it + 1);
+        }
+        // one to three tiles are left, `it` is even
+        const int left = n_tiles - it;
+        if (left == 3) {
+            tile(s0, yes, yes, it);
+            tile(s1, no, yes, it + 1);
+            tile(s0, no, no, it + 2);
+        } else if (left == 2) {
+            tile(s0, no, yes, it);
+            tile(s1, no, no, it + 1);
+        } else {
+            tile(s0, no, no, it);
+        }
     }
 
+    if (wave_active && p.splits > 1) {
+        // partial result of this slice: rows of the workgroup's 64, [HD] unnormalised output, m, l
+        float *base = p.part + ((((size_t)blockIdx.x * gridDim.y + blockIdx.y) * p.splits + blockIdx.z) * 64) * (HD + 2);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float *rowp = base + (size_t)(wave * 16 + 4 * kq + i) * (HD + 2);
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+                rowp[16 * db + c] = i == 0 ? o[db].x : i == 1 ? o[db].y : i == 2 ? o[db].z : o[db].w;
+        }
+        if (kq == 0) {
+            float *rowp = base + (size_t)(wave * 16 + c) * (HD + 2);
+            rowp[HD] = m_run;
+            rowp[HD + 1] = l_run;
+        }
+        return;
+    }
     if (wave_active) {
         float inv[4];
 #pragma unroll
@@ -261,12 +377,72 @@ __global__ __launch_bounds__(256) void paged_attn_kernel(const AttnParams p) {
     }
 }
 
+// Merge of the key slices: out[row] = sum_s exp2(m_s - m) O_s / sum_s exp2(m_s - m) l_s, slices in
+// order. One workgroup per (sequence, KV head, row group, 256 / HD rows): a thread owns one output
+// element and walks the slices, neighbouring threads reading neighbouring floats.
+template <typename T, int HD>
+__global__ __launch_bounds__(256) void paged_attn_merge_kernel(const AttnParams p) {
+    constexpr int RPW = 256 / HD;                       // rows per workgroup
+    const int seq = blockIdx.x / p.KVH, kvh = blockIdx.x % p.KVH;
+    const int Gq = p.H / p.KVH;
+    int ql = 1, q0 = seq;
+    if (p.q_lens) ql = p.q_lens[seq];
+    const int rows_total = ql * Gq;
+    const int r = (int)blockIdx.z * RPW + (int)threadIdx.x / HD, d = threadIdx.x % HD;
+    const int row = (int)blockIdx.y * 64 + r;
+    if (p.context_lens[seq] <= 0 || row >= rows_total) return;   // uniform per wavefront (HD >= 64)
+    if (p.q_lens) q0 = attn_first_token(p.q_lens, seq);
+    const float *base = p.part + ((((size_t)blockIdx.x * gridDim.y + blockIdx.y) * p.splits) * 64 + r) * (HD + 2);
+    const size_t stride = (size_t)64 * (HD + 2);
+    float m = -INFINITY;
+#pragma unroll 8
+    for (int s = 0; s < p.splits; ++s) m = fmaxf(m, base[s * stride + HD]);
+    if (m == -INFINITY) m = 0.0f;
+    float l = 0.0f, acc = 0.0f;
+#pragma unroll 8
+    for (int s = 0; s < p.splits; ++s) {
+        const float *rp = base + s * stride;
+        const float f = exp2f(rp[HD] - m);
+        l += f * rp[HD + 1];
+        acc += f * rp[d];
+    }
+    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+    const int tok = row / Gq, hq = row % Gq;
+    ((uint16_t *)p.out)[((size_t)(q0 + tok) * p.H + kvh * Gq + hq) * HD + d] = AttnT<T>::from_f32(acc * inv);
+}
+
+#ifndef ATTN_TARGET_WGS
+#define ATTN_TARGET_WGS 512
+#endif
+// key slices per sequence: enough workgroups to fill the chip, at least 8 tiles of keys each
+static int attn_splits(int n_seqs, int kvh, int row_groups, int max_blocks, int block_size) {
+    const long base = (long)n_seqs * kvh * row_groups;
+    const long max_tiles = ((long)max_blocks * block_size + 31) / 32;
+    long s = (ATTN_TARGET_WGS + base - 1) / base;
+    if (s > max_tiles / 8) s = max_tiles / 8;
+    if (s > 64) s = 64;
+    return s < 1 ? 1 : (int)s;
+}
+
+extern "C" size_t odsd_paged_attention_workspace_bytes(int32_t n_seqs, int32_t max_q_len, int32_t num_heads,
+                                                       int32_t num_kv_heads, int32_t head_dim,
+                                                       int32_t block_size, int32_t max_blocks) {
+    if (n_seqs <= 0 || max_q_len <= 0 || num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads ||
+        block_size <= 0 || max_blocks <= 0 || (head_dim != 64 && head_dim != 128))
+        return 0;
+    const int rg = (max_q_len * (num_heads / num_kv_heads) + 63) / 64;
+    const int splits = attn_splits(n_seqs, num_kv_heads, rg, max_blocks, block_size);
+    if (splits == 1) return 256;
+    return odsd_round_up((size_t)n_seqs * num_kv_heads * rg * splits * 64 * (head_dim + 2) * sizeof(float), 256);
+}
+
 extern "C" int odsd_paged_attention(const void *q, const void *k_cache, const void *v_cache,
                                     const int32_t *block_tables, const int32_t *context_lens,
                                     const int32_t *q_lens, int32_t n_seqs, int32_t max_q_len,
                                     int32_t num_heads, int32_t num_kv_heads, int32_t head_dim,
                                     int32_t block_size, int32_t max_blocks, int64_t num_slots,
-                                    float softmax_scale, int32_t dtype, void *out, void *stream) {
+                                    float softmax_scale, int32_t dtype, void *out, void *workspace,
+                                    size_t workspace_bytes, void *stream) {
     if (n_seqs < 0 || max_q_len <= 0 || num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads ||
         block_size <= 0 || max_blocks <= 0 || num_slots <= 0)
         return ODSD_ERR_SHAPE;
@@ -282,16 +458,33 @@ extern "C" int odsd_paged_attention(const void *q, const void *k_cache, const vo
     p.n_seqs = n_seqs; p.H = num_heads; p.KVH = num_kv_heads; p.max_blocks = max_blocks;
     p.block_size = block_size; p.num_slots = num_slots;
     p.scale_log2e = softmax_scale * 1.4426950408889634f;
-    const int rows_max = max_q_len * (num_heads / num_kv_heads);
-    const dim3 grid((unsigned)(n_seqs * num_kv_heads), (unsigned)((rows_max + 63) / 64));
-    hipStream_t st = (hipStream_t)stream;
-    if (dtype == ODSD_DT_F16) {
-        if (head_dim == 128) paged_attn_kernel<half_t, 128><<<grid, 256, 0, st>>>(p);
-        else paged_attn_kernel<half_t, 64><<<grid, 256, 0, st>>>(p);
-    } else {
-        if (head_dim == 128) paged_attn_kernel<__bf16, 128><<<grid, 256, 0, st>>>(p);
-        else paged_attn_kernel<__bf16, 64><<<grid, 256, 0, st>>>(p);
+    const int rg = (max_q_len * (num_heads / num_kv_heads) + 63) / 64;
+    p.splits = attn_splits(n_seqs, num_kv_heads, rg, max_blocks, block_size);
+    if (p.splits > 1) {
+        const size_t need = odsd_paged_attention_workspace_bytes(n_seqs, max_q_len, num_heads, num_kv_heads,
+                                                                 head_dim, block_size, max_blocks);
+        if (!workspace) return ODSD_ERR_NULL;
+        if (!odsd_aligned16(workspace)) return ODSD_ERR_ALIGN;
+        if (workspace_bytes < need) return ODSD_ERR_WORKSPACE;
+        p.part = (float *)workspace;
     }
+    const dim3 grid((unsigned)(n_seqs * num_kv_heads), (unsigned)rg, (unsigned)p.splits);
+    const dim3 mgrid((unsigned)(n_seqs * num_kv_heads), (unsigned)rg, (unsigned)(64 / (256 / head_dim)));
+    hipStream_t st = (hipStream_t)stream;
+#define ATTN_GO(T, HDV)                                                              \
+    do {                                                                             \
+        if (block_size % 32 == 0) paged_attn_kernel<T, HDV, true><<<grid, 256, 0, st>>>(p);  \
+        else paged_attn_kernel<T, HDV, false><<<grid, 256, 0, st>>>(p);              \
+        if (p.splits > 1) paged_attn_merge_kernel<T, HDV><<<mgrid, 256, 0, st>>>(p); \
+    } while (0)
+    if (dtype == ODSD_DT_F16) {
+        if (head_dim == 128) ATTN_GO(half_t, 128);
+        else ATTN_GO(half_t, 64);
+    } else {
+        if (head_dim == 128) ATTN_GO(__bf16, 128);
+        else ATTN_GO(__bf16, 64);
+    }
+#undef ATTN_GO
     ODSD_CHECK_LAUNCH();
     return ODSD_OK;
 }

@@ -82,11 +82,18 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         return out
     scale = head_dim ** -0.5 if softmax_scale is None else softmax_scale
     lib = _lib.load()
+    mq = max_q_len or n_tokens
+    nbytes = lib.odsd_paged_attention_workspace_bytes(n_seqs, mq, num_heads, num_kv_heads, head_dim, block_size,
+                                                      tables.shape[1])
+    if nbytes == 0:
+        raise _lib.OdsdError("paged attention: unsupported shape (head_dim 64 or 128, heads a multiple of KV heads)")
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
     _lib.check(lib.odsd_paged_attention(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), tables.data_ptr(),
                                         lens.data_ptr(), None if q_lens is None else q_lens.data_ptr(), n_seqs,
-                                        max_q_len or n_tokens, num_heads, num_kv_heads, head_dim, block_size,
+                                        mq, num_heads, num_kv_heads, head_dim, block_size,
                                         tables.shape[1], k_cache.numel() // D, scale, dt, out.data_ptr(),
-                                        torch.cuda.current_stream().cuda_stream), "odsd_paged_attention")
+                                        ws.data_ptr(), nbytes, torch.cuda.current_stream().cuda_stream),
+               "odsd_paged_attention")
     return out
 
 

@@ -83,6 +83,23 @@ def test_argument_checks_need_no_gpu():
     assert lib.odsd_kv_store(1 << 20, 1 << 20, 32, 64, 1 << 20, 1 << 20, 1 << 20, None, 4, 4, 64, 2, 16, None) == 2
     assert lib.odsd_kv_store(1 << 20, 1 << 20, 64, 64, 1 << 20, 1 << 20, 1 << 20, None, 4, 4, 64, 3, 16, None) == 7
     assert lib.odsd_kv_store(None, None, 64, 64, None, None, None, None, 0, 0, 64, 2, 16, None) == 0
+    # paged attention: argument checks (q, k, v, tables, lens, q_lens, n_seqs, max_q_len, H, KVH, HD, block,
+    # max_blocks, num_slots, scale, dtype, out, workspace, workspace_bytes, stream)
+    P = 1 << 20
+    att = lambda *a: lib.odsd_paged_attention(*a)
+    assert att(P, P, P, P, P, None, 2, 8, 32, 4, 128, 256, 16, 8192, 0.1, _lib.DT_BF16, None, None, 0, None) == 1
+    assert att(P, P, P, P, P, None, 2, 8, 32, 5, 128, 256, 16, 8192, 0.1, _lib.DT_BF16, P, None, 0, None) == 2
+    assert att(P, P, P, P, P, None, 2, 8, 32, 4, 96, 256, 16, 8192, 0.1, _lib.DT_BF16, P, None, 0, None) == 3
+    assert att(P, P, P, P, P, None, 2, 8, 32, 4, 128, 256, 16, 8192, 0.1, 9, P, None, 0, None) == 7
+    assert att(None, None, None, None, None, None, 0, 8, 32, 4, 128, 256, 16, 8192, 0.1, _lib.DT_BF16, None, None, 0, None) == 0
+    # few sequences with long tables share a sequence's keys between workgroups: workspace required
+    need = lib.odsd_paged_attention_workspace_bytes(2, 8, 32, 4, 128, 256, 16)
+    assert need > 256 and need % 256 == 0
+    assert att(P, P, P, P, P, None, 2, 8, 32, 4, 128, 256, 16, 8192, 0.1, _lib.DT_BF16, P, None, 0, None) == 1
+    assert att(P, P, P, P, P, None, 2, 8, 32, 4, 128, 256, 16, 8192, 0.1, _lib.DT_BF16, P, P, need - 1, None) == 5
+    assert lib.odsd_paged_attention_workspace_bytes(2, 8, 32, 4, 96, 256, 16) == 0
+    # many sequences: one workgroup per (sequence, KV head) walks all its keys, no partial results
+    assert lib.odsd_paged_attention_workspace_bytes(512, 1, 32, 4, 128, 256, 16) == 256
     empty = _lib.MoeShape(0, 256, 8, 2, 256, 1, _lib.DT_BF16, 0)       # T == 0 is a no-op
     assert lib.odsd_dispatch(C.byref(empty), 1 << 20, 1 << 20, 1 << 20, 1 << 20, 1 << 20, 1 << 20, None) == 0
 

@@ -72,6 +72,9 @@ ATTN_CASES = [
     (torch.float16, 8, 8, 64, 8, [(95, 4), (1, 1), (33, 2)]),                             # no grouping, head_dim 64
     (torch.bfloat16, 16, 2, 128, 16, [(260, 12), (64, 9)]),                               # 96 and 72 query rows: two row groups
     (torch.float16, 32, 4, 128, 32, [(513, None), (40, None), (1, None), (250, None)]),   # decode step
+    (torch.bfloat16, 32, 4, 128, 256, [(5000, 8)]),                                       # one long sequence: 19 key slices
+    (torch.float16, 16, 8, 64, 64, [(3000, 4), (100, 4), (2977, 1)]),                     # slices with ragged ends, head_dim 64
+    (torch.bfloat16, 32, 4, 128, 48, [(1500, 6), (700, 2)]),                              # block size not a multiple of the key tile
 ]
 
 
