@@ -19,6 +19,7 @@ Every result carries
     over the same inputs, with fp32 weights dequantised beforehand.
 """
 import argparse
+import dataclasses
 import json
 import os
 import sys
@@ -266,7 +267,7 @@ def bench_stack(wl, dev, steps, warmup, with_cpu, cpu_layers=4):
         "layer_hbm_frac": round(alg_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
         "kernel_ms": {n: round(v, 5) for n, v in k.items()},
         "kernel_ms_sum": round(sum(stage_ms), 5),
-        "kernel_ms_note": "sums over the 48 layers of one step",
+        "kernel_ms_note": f"sums over the {wl.layers} layers of one step",
         # the dominant kernel runs once per layer: average launch = sum over layers / layers
         "roofline": _roofline(wl, k["gate_up"] / wl.layers, gu_bytes_total / wl.layers),
     }
@@ -370,6 +371,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default=None, help="measure this configuration only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
+    ap.add_argument("--layers", type=int, default=None,
+                    help="stack workloads: run this many layers instead of the configuration's (hardware-counter "
+                         "runs, where every dispatch is costly; a kernel's per-launch figures do not depend on it)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (use --gpus 1)", file=sys.stderr)
@@ -383,6 +387,11 @@ def main():
     torch.cuda.set_device(dev)
 
     head = CONFIGS[args.workload or HEADLINE]
+    if args.layers is not None:
+        if head.layers <= 1 or args.layers < 1:
+            print("--layers applies to a stack workload and must be positive", file=sys.stderr)
+            sys.exit(2)
+        head = dataclasses.replace(head, layers=args.layers)
     main_res = run_workload(head, dev, args.steps, args.warmup, not args.no_cpu)
     line = {
         "metric": "int4 MoE-layer tokens/s", "value": main_res["tokens_per_s"], "unit": "tokens/s",

@@ -222,7 +222,7 @@ int odsd_kv_store(const void *key, const void *value, int64_t key_stride, int64_
  *                block_tables[s][p / block_size] * block_size + p % block_size
  *   context_lens [n_seqs]: cached tokens of the sequence INCLUDING this step's (stored before)
  *   query j of sequence s attends positions 0 .. context_lens[s] - q_lens[s] + j; query head h
- *   reads KV head h / (num_heads / num_kv_heads); scores scaled by softmax_scale; fp32 softmax
+ *   reads KV head h / (num_heads / num_kv_heads); scores scaled by softmax_scale (> 0); fp32 softmax
  *   out          [n_tokens, num_heads, head_dim] in the dtype of q (ODSD_DT_BF16 or ODSD_DT_F16)
  * max_q_len: an upper bound of q_lens (sizes the launch); head_dim 64 or 128.
  * workspace: odsd_paged_attention_workspace_bytes(...) bytes (with few sequences the keys of one

@@ -48,6 +48,12 @@ template <> struct AttnT<half_t> {
         return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
     }
     __device__ static __forceinline__ uint16_t from_f32(float v) { return __builtin_bit_cast(uint16_t, (half_t)v); }
+    // two values, round to nearest even, as one 32-bit word (a in the low half)
+    __device__ static __forceinline__ uint32_t pack2(float a, float b) {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        typedef float f2 __attribute__((ext_vector_type(2)));
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f2{a, b}, h2));
+    }
 };
 template <> struct AttnT<__bf16> {
     typedef bf16x8_t V8;
@@ -55,6 +61,11 @@ template <> struct AttnT<__bf16> {
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
     }
     __device__ static __forceinline__ uint16_t from_f32(float v) { return f32_to_bf16(v); }
+    __device__ static __forceinline__ uint32_t pack2(float a, float b) {   // v_cvt_pk_bf16_f32
+        typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+        typedef float f2 __attribute__((ext_vector_type(2)));
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f2{a, b}, b2));
+    }
 };
 
 // position of key `key` (0..31) of a tile inside a row of the transposed V tile: the 8 keys a
@@ -78,17 +89,16 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
     constexpr int VT_LD = 40;            // halfs per row of the transposed V tile (32 keys + pad)
     constexpr int PIECES = 32 * (HD / 8) / 256;   // 16-byte pieces of a V tile per thread
     __shared__ __attribute__((aligned(16))) uint16_t vt[2][HD * VT_LD];
+    // K tile as stored ([key][HD]), 16-byte pieces of a row XORed with the key so that the 16 lanes
+    // reading the same piece of 16 different keys hit different banks
+    __shared__ __attribute__((aligned(16))) uint16_t kt[2][32 * HD];
 
     const int seq = blockIdx.x / p.KVH, kvh = blockIdx.x % p.KVH;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int c = lane & 15, kq = lane >> 4;
     const int Gq = p.H / p.KVH;
     const int L = p.context_lens[seq];
-    int ql = 1, q0 = seq;
-    if (p.q_lens) {
-        ql = p.q_lens[seq];
-        q0 = attn_first_token(p.q_lens, seq);
-    }
+    const int ql = p.q_lens ? p.q_lens[seq] : 1;
     const int rows_total = ql * Gq;
     if (L <= 0 || ql <= 0 || (int)blockIdx.y * 64 >= rows_total) return;
     const int row0 = ((int)blockIdx.y * 4 + wave) * 16;
@@ -97,12 +107,16 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
     const uint16_t *kc = (const uint16_t *)p.k_cache, *vc = (const uint16_t *)p.v_cache;
     const int32_t *bt = p.block_tables + (size_t)seq * p.max_blocks;
 
-    // this lane's query row (B operand of S^T = K Q^T: lane (c, kq) holds Q[row c][32 j + 8 kq ..])
+    // this lane's query row (B operand of S^T = K Q^T: lane (c, kq) holds Q[row c][32 j + 8 kq ..]);
+    // fetched after the first K / V tiles are on their way (the first token of the sequence is a
+    // prefix sum over the query lengths: a dependent chain that nothing else waits for)
     const int row = row0 + c;
     const bool row_ok = wave_active && row < rows_total;
     const int tok = row_ok ? row / Gq : 0, hq = row_ok ? row % Gq : 0;
     V8 qf[NJ];
-    {
+    int q0 = seq;
+    auto load_q = [&]() {
+        if (p.q_lens) q0 = attn_first_token(p.q_lens, seq);
         const uint16_t *qp = (const uint16_t *)p.q + ((size_t)(q0 + tok) * p.H + kvh * Gq + hq) * HD + 8 * kq;
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
@@ -110,26 +124,35 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
             if (row_ok) raw = *(const uint4_t *)(qp + 32 * j);
             qf[j] = __builtin_bit_cast(V8, raw);
         }
-    }
+    };
     const int kmax = row_ok ? L - ql + tok : -1;      // last position this row attends
+    int kmin_wave = row_ok ? kmax : 0x7fffffff;        // tiles ending at or before it need no mask
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) kmin_wave = min(kmin_wave, __shfl_xor(kmin_wave, d, ODSD_WAVE));
+    const float sc = p.scale_log2e;
 
-    float m_run = -INFINITY, l_run = 0.0f;             // per query row c (replicated over kq)
+    // per query row c: the reference point of its exponentials (the same in its 4 kq lanes) and
+    // this lane's share of the sum of its probabilities
+    float m_run = -INFINITY, l_run = 0.0f;
     float4_t o[NDB];
 #pragma unroll
     for (int db = 0; db < NDB; ++db) o[db] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    // Software pipeline over the 32-key tiles, two tiles deep: during tile `it` the K fragments and
-    // V pieces of tile it + 2 are fetched into the register set tile `it` has just finished with,
-    // V of tile it + 1 goes transposed into the other LDS buffer, and the block-table entries of
-    // tile it + 3 are requested BEFORE the fetches (the load counter retires in order: a younger
-    // table read awaited by the next tile would otherwise drain the big fetches issued before it).
-    // The steady-state tiles fetch unconditionally and the last two tiles are compiled without the
-    // fetch, so that no wait is placed after a join of "fetched" and "did not fetch".
-    //   K: lane (c, kq) reads 16 bytes of key row 16 t + c for each 32-dim step (the A operand)
-    //   V: piece = tid + 256 u -> key = piece / (HD / 8), dims 8 * (piece % (HD / 8)) ..
+    // Software pipeline over the 32-key tiles, two tiles deep.  A tile's K and V rows are fetched
+    // once per workgroup, 16 bytes per thread and piece (piece = tid + 256 u -> key = piece /
+    // (HD / 8), dims 8 * (piece % (HD / 8)) ..), two tiles ahead into one of two register sets;
+    // one tile ahead they go to LDS -- K as stored, V transposed -- and every wavefront reads its
+    // MFMA operands from there (K fetched per wavefront instead costs four times the L2 traffic
+    // and was what bounded the kernel).  During tile `it`: the set that held tile `it` is refilled
+    // with tile it + 2, the other set (tile it + 1) goes to the other LDS buffers, and the
+    // block-table entries of tile it + 3 are requested BEFORE the fetches (the load counter retires
+    // in order: a younger table read awaited by the next tile would otherwise drain the big
+    // fetches issued before it).  The steady-state tiles fetch unconditionally and the last two
+    // tiles are compiled without the fetch, so that no wait is placed after a join of "fetched"
+    // and "did not fetch".
     // ALIGNED (block_size a multiple of 32): a tile lies in one cache block, so its table entry is
-    // one wavefront-uniform read; otherwise every lane reads the entry of its own key.
-    constexpr int NE = ALIGNED ? 1 : 2 + PIECES;        // table entries a tile needs per lane
+    // one wavefront-uniform read; otherwise every lane reads the entries of its own keys.
+    constexpr int NE = ALIGNED ? 1 : PIECES;            // table entries a tile needs per lane
     const int k_last = L - 1;
     const int bs = p.block_size;
     auto entry_at = [&](int pos) -> int32_t { return bt[min(min(pos, k_last) / bs, p.max_blocks - 1)]; };
@@ -138,9 +161,7 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
             e[0] = entry_at(k0);
         } else {
 #pragma unroll
-            for (int t = 0; t < 2; ++t) e[t] = entry_at(k0 + 16 * t + c);
-#pragma unroll
-            for (int u = 0; u < PIECES; ++u) e[2 + u] = entry_at(k0 + (tid + 256 * u) / (HD / 8));
+            for (int u = 0; u < PIECES; ++u) e[u] = entry_at(k0 + (tid + 256 * u) / (HD / 8));
         }
     };
     // slot of position pos (clamped into the sequence) in the block whose table entry is b; an
@@ -151,7 +172,7 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
         const int64_t sl = (int64_t)b * bs + (pc - blk * bs);
         return (b >= 0 && blk < p.max_blocks && sl < p.num_slots) ? sl : 0;
     };
-    uint4_t kreg[2][2][NJ], vreg[2][PIECES];
+    uint4_t kreg[2][PIECES], vreg[2][PIECES];
     // fetch of the tile at k0, whose table entries are e
     auto fetch = [&](auto set, int k0, const int32_t (&e)[NE]) {
         constexpr int S = decltype(set)::value;
@@ -167,36 +188,26 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
             const size_t base = (size_t)slot0 * D + kvh * HD;
             const uint16_t *kb = kc + base, *vb = vc + base;
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                const uint32_t off = (uint32_t)min(16 * t + c, lim) * (uint32_t)D + 8 * kq;
-#pragma unroll
-                for (int j = 0; j < NJ; ++j) kreg[S][t][j] = *(const uint4_t *)(kb + off + 32 * j);
-            }
-#pragma unroll
             for (int u = 0; u < PIECES; ++u) {
                 const int piece = tid + 256 * u;
                 const uint32_t off = (uint32_t)min(piece / (HD / 8), lim) * (uint32_t)D + 8 * (piece % (HD / 8));
+                kreg[S][u] = *(const uint4_t *)(kb + off);
                 vreg[S][u] = *(const uint4_t *)(vb + off);
             }
         } else {
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                const int64_t sl = slot_in(e[t], k0 + 16 * t + c);
-                const uint16_t *kp = kc + sl * D + kvh * HD + 8 * kq;
-#pragma unroll
-                for (int j = 0; j < NJ; ++j) kreg[S][t][j] = *(const uint4_t *)(kp + 32 * j);
-            }
-#pragma unroll
             for (int u = 0; u < PIECES; ++u) {
                 const int piece = tid + 256 * u;
-                const int64_t sl = slot_in(e[2 + u], k0 + piece / (HD / 8));
-                vreg[S][u] = *(const uint4_t *)(vc + sl * D + kvh * HD + 8 * (piece % (HD / 8)));
+                const int64_t sl = slot_in(e[u], k0 + piece / (HD / 8));
+                const size_t off = (size_t)sl * D + kvh * HD + 8 * (piece % (HD / 8));
+                kreg[S][u] = *(const uint4_t *)(kc + off);
+                vreg[S][u] = *(const uint4_t *)(vc + off);
             }
         }
     };
     // V^T tile in LDS: row = dim, 32 key positions (+ pad); the 8-position segment index is XORed
     // with (dim / 8) & 3 so that the 16 lanes writing one key's 16 dim chunks spread over the banks
-    auto store_v = [&](auto set, int buf) {
+    auto store_kv = [&](auto set, int buf) {
         constexpr int S = decltype(set)::value;
 #pragma unroll
         for (int u = 0; u < PIECES; ++u) {
@@ -207,6 +218,7 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
 #pragma unroll
             for (int i = 0; i < 8; ++i)
                 vt[buf][(8 * ch + i) * VT_LD + pos] = (uint16_t)(w[i >> 1] >> (16 * (i & 1)));
+            *(uint4_t *)&kt[buf][key * HD + 8 * (ch ^ (key & (HD / 8 - 1)))] = kreg[S][u];
         }
     };
 
@@ -218,7 +230,7 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
     const int kbase = t_begin * 32;
     int32_t pend[NE];                                   // entries of the tile after the newest fetched one
 
-    // one tile; S: the register set holding its K. FETCH: tile it + 2 exists and is fetched (and
+    // one tile; S: the register set that held it (free now). FETCH: tile it + 2 exists and is fetched (and
     // the entries of tile it + 3 requested); STORE: tile it + 1 exists and its V goes to LDS
     auto tile = [&](auto set, auto fetch_c, auto store_c, int it) {
         constexpr int S = decltype(set)::value;
@@ -231,8 +243,11 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
             for (int t = 0; t < 2; ++t) {
                 float4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int j = 0; j < NJ; ++j)
-                    acc = AttnT<T>::mfma(__builtin_bit_cast(V8, kreg[S][t][j]), qf[j], acc);
+                for (int j = 0; j < NJ; ++j) {
+                    const int key = 16 * t + c;
+                    const uint4_t kraw = *(const uint4_t *)&kt[buf][key * HD + 8 * ((4 * j + kq) ^ (key & (HD / 8 - 1)))];
+                    acc = AttnT<T>::mfma(__builtin_bit_cast(V8, kraw), qf[j], acc);
+                }
                 st[t] = acc;
             }
         }
@@ -244,53 +259,44 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
             fetch(set, k0 + 64, now);
         }
         if (wave_active) {
-            // lane (c, kq) holds keys k0 + 16 t + 4 kq + i of query row c: mask, running max and sum
-            float sv[8];
-            float mx = -INFINITY;
+            // lane (c, kq) holds keys k0 + 16 t + 4 kq + i of query row c (raw scores, before the
+            // softmax scale).  Only tiles that reach past the first row's last key need the mask.
+            float a[8] = {st[0].x, st[0].y, st[0].z, st[0].w, st[1].x, st[1].y, st[1].z, st[1].w};
+            if (k0 + 31 > kmin_wave) {
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                const float a[4] = {st[t].x, st[t].y, st[t].z, st[t].w};
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int pos = k0 + 16 * t + 4 * kq + i;
-                    const float v = pos <= kmax ? a[i] * p.scale_log2e : -INFINITY;
-                    sv[4 * t + i] = v;
-                    mx = fmaxf(mx, v);
-                }
+                for (int i = 0; i < 8; ++i)
+                    a[i] = k0 + 16 * (i >> 2) + 4 * kq + (i & 3) <= kmax ? a[i] : -INFINITY;
             }
-            mx = fmaxf(mx, __shfl_xor(mx, 16, ODSD_WAVE));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, ODSD_WAVE));
-            const float m_new = fmaxf(m_run, mx);
-            // a row with nothing to attend yet keeps m = -inf: use 0 as the reference point then
-            const float m_ref = m_new == -INFINITY ? 0.0f : m_new;
-            const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);        // m_run = -inf -> 0
-            float ps = 0.0f;
-            uint16_t pb[8];
+            float mx = fmaxf(fmaxf(fmaxf(a[0], a[1]), fmaxf(a[2], a[3])), fmaxf(fmaxf(a[4], a[5]), fmaxf(a[6], a[7])));
+            // The reference point m_run of a row moves only when some score of the wavefront
+            // exceeds it by more than 2^8 (probabilities up to 256 are as exact in fp16 / bf16 as
+            // those below 1, and the sums are fp32): most tiles then need no exchange between
+            // lanes at all -- no maximum, no rescaling of the output, no sum (l_run stays a
+            // per-lane partial sum until the end).
+            if (__any(mx * sc > m_run + 8.0f)) {
+                mx = fmaxf(mx, __shfl_xor(mx, 16, ODSD_WAVE));
+                mx = fmaxf(mx, __shfl_xor(mx, 32, ODSD_WAVE));
+                const float m_new = fmaxf(m_run, mx * sc);
+                // a row with nothing to attend yet keeps m = -inf: use 0 as the reference point then
+                const float alpha = __builtin_amdgcn_exp2f(m_run - (m_new == -INFINITY ? 0.0f : m_new));   // m_run = -inf -> 0
+                l_run *= alpha;
+                m_run = m_new;
+                // the output tile holds rows 4 kq + i in lane (dim, kq): fetch those rows' alpha
+                float al[4];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const float e = __builtin_amdgcn_exp2f(sv[i] - m_ref);         // masked -> 0
-                pb[i] = AttnT<T>::from_f32(e);
-                ps += e;
-            }
-            ps += __shfl_xor(ps, 16, ODSD_WAVE);
-            ps += __shfl_xor(ps, 32, ODSD_WAVE);
-            l_run = l_run * alpha + ps;
-            m_run = m_new;
-            const V8 pf = __builtin_bit_cast(V8, uint4_t{(uint32_t)pb[0] | ((uint32_t)pb[1] << 16),
-                                                          (uint32_t)pb[2] | ((uint32_t)pb[3] << 16),
-                                                          (uint32_t)pb[4] | ((uint32_t)pb[5] << 16),
-                                                          (uint32_t)pb[6] | ((uint32_t)pb[7] << 16)});
-            // the output tile holds rows 4 kq + i in lane (dim, kq): fetch those rows' alpha
-            float al[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) al[i] = __shfl(alpha, 4 * kq + i, ODSD_WAVE);
-            // once the running maxima have settled no row of the wavefront rescales any more
-            if (__any(alpha != 1.0f)) {
+                for (int i = 0; i < 4; ++i) al[i] = __shfl(alpha, 4 * kq + i, ODSD_WAVE);
 #pragma unroll
                 for (int db = 0; db < NDB; ++db) {
                     o[db].x *= al[0]; o[db].y *= al[1]; o[db].z *= al[2]; o[db].w *= al[3];
                 }
             }
+            const float neg_ref = m_run == -INFINITY ? 0.0f : -m_run;
+            float pe[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) pe[i] = __builtin_amdgcn_exp2f(fmaf(a[i], sc, neg_ref));   // masked -> 0
+            l_run += ((pe[0] + pe[1]) + (pe[2] + pe[3])) + ((pe[4] + pe[5]) + (pe[6] + pe[7]));
+            const V8 pf = __builtin_bit_cast(V8, uint4_t{AttnT<T>::pack2(pe[0], pe[1]), AttnT<T>::pack2(pe[2], pe[3]),
+                                                          AttnT<T>::pack2(pe[4], pe[5]), AttnT<T>::pack2(pe[6], pe[7])});
 #pragma unroll
             for (int db = 0; db < NDB; ++db) {
                 const int seg = kq ^ ((2 * db + (c >> 3)) & 3);
@@ -298,8 +304,8 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
                 o[db] = AttnT<T>::mfma(pf, vf, o[db]);
             }
         }
-        // V of tile it + 1 (other set, fetched during tile it - 1) into the other LDS buffer
-        if constexpr (STORE) store_v(std::integral_constant<int, S ^ 1>{}, buf ^ 1);
+        // K and V of tile it + 1 (other set, fetched during tile it - 1) into the other LDS buffers
+        if constexpr (STORE) store_kv(std::integral_constant<int, S ^ 1>{}, buf ^ 1);
         __syncthreads();
     };
 
@@ -308,7 +314,7 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
         const std::integral_constant<int, 1> s1;
         const std::true_type yes;
         const std::false_type no;
-        // prologue: tiles 0 and 1 fetched, V of tile 0 in LDS, the entries of tile 2 requested
+        // prologue: tiles 0 and 1 fetched, tile 0 in LDS, the entries of tile 2 requested
         request(kbase, pend);
         fetch(s0, kbase, pend);
         if (n_tiles > 1) {
@@ -316,7 +322,8 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
             fetch(s1, kbase + 32, pend);
         }
         request(kbase + 64, pend);
-        store_v(s0, 0);
+        load_q();
+        store_kv(s0, 0);
         __syncthreads();
         int it = 0;
         for (; it + 3 < n_tiles; it += 2) {
@@ -337,6 +344,8 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
         }
     }
 
+    l_run += __shfl_xor(l_run, 16, ODSD_WAVE);
+    l_run += __shfl_xor(l_run, 32, ODSD_WAVE);
     if (wave_active && p.splits > 1) {
         // partial result of this slice: rows of the workgroup's 64, [HD] unnormalised output, m, l
         float *base = p.part + ((((size_t)blockIdx.x * gridDim.y + blockIdx.y) * p.splits + blockIdx.z) * 64) * (HD + 2);
@@ -444,7 +453,7 @@ extern "C" int odsd_paged_attention(const void *q, const void *k_cache, const vo
                                     float softmax_scale, int32_t dtype, void *out, void *workspace,
                                     size_t workspace_bytes, void *stream) {
     if (n_seqs < 0 || max_q_len <= 0 || num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads ||
-        block_size <= 0 || max_blocks <= 0 || num_slots <= 0)
+        block_size <= 0 || max_blocks <= 0 || num_slots <= 0 || !(softmax_scale > 0.0f))
         return ODSD_ERR_SHAPE;
     if (head_dim != 64 && head_dim != 128) return ODSD_ERR_UNSUPPORTED;
     if (dtype != ODSD_DT_BF16 && dtype != ODSD_DT_F16) return ODSD_ERR_DTYPE;
