@@ -277,6 +277,83 @@ def bench_stack(wl, dev, steps, warmup, with_cpu, cpu_layers=4):
     return res
 
 
+def bench_attention(dev, steps, warmup, with_cpu):
+    """The step on the other side of the MoE block in a verify pass: the draft tokens' K / V rows are
+    scattered into the paged cache and every query attends its sequence's cached keys (Qwen3-30B-A3B
+    heads: 32 query / 4 KV heads of 128; 32 sequences x 8 draft tokens, 2048 cached tokens each,
+    256-token cache blocks in random order).  Timed as replays of a HIP graph holding one store +
+    one attention call, so that the Python wrapper's host time is not in the figure."""
+    import torch
+    import on_device_sd_amd as odsd
+    name = "qwen3_30b_verify_attention_s32_q8_ctx2048"
+    H, KVH, HD, bs, n_seqs, ql, L = 32, 4, 128, 256, 32, 8, 2048
+    _log(f"{name}: building the cache")
+    nb = L // bs
+    g = torch.Generator().manual_seed(0)
+    tables = torch.randperm(n_seqs * nb, generator=g).view(n_seqs, nb).to(torch.int32)
+    k_cache = torch.randn(n_seqs * nb * bs, KVH * HD, generator=g).to(torch.bfloat16).to(dev)
+    v_cache = torch.randn(n_seqs * nb * bs, KVH * HD, generator=g).to(torch.bfloat16).to(dev)
+    q = torch.randn(n_seqs * ql, H, HD, generator=g).to(torch.bfloat16).to(dev)
+    k_new = torch.randn(n_seqs * ql, KVH, HD, generator=g).to(torch.bfloat16).to(dev)
+    v_new = torch.randn(n_seqs * ql, KVH, HD, generator=g).to(torch.bfloat16).to(dev)
+    pos = torch.arange(L - ql, L)
+    slots = (tables[:, (pos // bs)].to(torch.int64) * bs + (pos % bs)).reshape(-1).to(torch.int32).to(dev)
+    ctx = {"block_tables": tables.to(dev), "context_lens": torch.full((n_seqs,), L, dtype=torch.int32, device=dev),
+           "verify_query_lens": torch.full((n_seqs,), ql, dtype=torch.int32, device=dev), "slot_mapping": slots}
+
+    def step():
+        odsd.store_kvcache(k_new, v_new, k_cache, v_cache, slots)
+        return odsd.paged_attention(q, k_cache, v_cache, ctx, KVH, bs, max_q_len=ql)
+
+    def timed(fn):
+        for _ in range(max(3, warmup)):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / steps
+
+    eager_ms = timed(step)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = step()
+    graph_ms = timed(graph.replay)
+    g_attn = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g_attn):
+        odsd.paged_attention(q, k_cache, v_cache, ctx, KVH, bs, max_q_len=ql)
+    attn_ms = timed(g_attn.replay)
+    kv_bytes = 2 * n_seqs * L * KVH * HD * 2 + 2 * q.numel() * 2
+    ach = kv_bytes / (attn_ms * 1e-3) / 1e9
+    n_tok = n_seqs * ql
+    res = {
+        "workload": name, "kind": "kv-cache store + paged causal attention (one layer of a verify step)",
+        "sequences": n_seqs, "query_tokens_per_sequence": ql, "context_len": L, "heads": H, "kv_heads": KVH,
+        "head_dim": HD, "block_size": bs, "tokens_per_s": round(n_tok / (graph_ms * 1e-3), 1),
+        "ms_per_step": round(graph_ms, 5), "ms_per_step_eager_python": round(eager_ms, 5),
+        "roofline": {"bound": "hbm", "kernel": "paged_attn_kernel + paged_attn_merge_kernel", "achieved": round(ach, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None,
+                     "algorithmic_bytes": kv_bytes, "kernel_ms": round(attn_ms, 5)},
+    }
+    if with_cpu:
+        # the oracle's restatement of the reference's fallback attention on a sample of the sequences
+        from oracle import moe_oracle as oracle
+        n_s = 4
+        qs = q[:n_s * ql].float().cpu()
+        kc, vc = k_cache.float().cpu(), v_cache.float().cpu()
+        cl = [L] * n_s
+        torch.set_num_threads(_host_threads())
+
+        def run():
+            oracle.paged_attention(qs, kc, vc, tables[:n_s], cl, [ql] * n_s, KVH, bs, HD ** -0.5)
+        sec, _ = _time_cpu(run, 10.0)
+        res["cpu_baseline"] = {"value": round(n_s * ql / sec, 1), "unit": "tokens/s", "cores": _host_threads(),
+                               "kind": "port", "sample": f"{n_s} of the {n_seqs} sequences (fp32 gather + matmul "
+                               "attention per sequence, the reference's fallback path), tokens/s of the sample"}
+    return res
+
+
 def _stack_active_experts(stack, x, wl):
     """Experts with at least one token, per layer, from the counts the whole-block call returns."""
     import torch
@@ -386,6 +463,9 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if args.workload == "attention":
+        print(json.dumps(bench_attention(dev, args.steps, args.warmup, not args.no_cpu)))
+        return
     head = CONFIGS[args.workload or HEADLINE]
     if args.layers is not None:
         if head.layers <= 1 or args.layers < 1:
@@ -409,6 +489,7 @@ def main():
     if args.workload is None:
         line["workloads"] = [run_workload(CONFIGS[name], dev, args.steps, args.warmup, not args.no_cpu)
                              for name in OTHERS]
+        line["workloads"].append(bench_attention(dev, args.steps, args.warmup, not args.no_cpu))
     print(json.dumps(line))
 
 

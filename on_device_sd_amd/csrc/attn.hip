@@ -388,36 +388,61 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
 
 // Merge of the key slices: out[row] = sum_s exp2(m_s - m) O_s / sum_s exp2(m_s - m) l_s, slices in
 // order. One workgroup per (sequence, KV head, row group, 256 / HD rows): a thread owns one output
-// element and walks the slices, neighbouring threads reading neighbouring floats.
+// element and walks the slices, neighbouring threads reading neighbouring floats.  (More rows per
+// workgroup, taken in turn, measured slower: each turn is one more exposed load latency.)
 template <typename T, int HD>
 __global__ __launch_bounds__(256) void paged_attn_merge_kernel(const AttnParams p) {
     constexpr int RPW = 256 / HD;                       // rows per workgroup
     const int seq = blockIdx.x / p.KVH, kvh = blockIdx.x % p.KVH;
     const int Gq = p.H / p.KVH;
-    int ql = 1, q0 = seq;
-    if (p.q_lens) ql = p.q_lens[seq];
+    const int ql = p.q_lens ? p.q_lens[seq] : 1;
     const int rows_total = ql * Gq;
-    const int r = (int)blockIdx.z * RPW + (int)threadIdx.x / HD, d = threadIdx.x % HD;
-    const int row = (int)blockIdx.y * 64 + r;
-    if (p.context_lens[seq] <= 0 || row >= rows_total) return;   // uniform per wavefront (HD >= 64)
-    if (p.q_lens) q0 = attn_first_token(p.q_lens, seq);
-    const float *base = p.part + ((((size_t)blockIdx.x * gridDim.y + blockIdx.y) * p.splits) * 64 + r) * (HD + 2);
-    const size_t stride = (size_t)64 * (HD + 2);
-    float m = -INFINITY;
-#pragma unroll 8
-    for (int s = 0; s < p.splits; ++s) m = fmaxf(m, base[s * stride + HD]);
-    if (m == -INFINITY) m = 0.0f;
-    float l = 0.0f, acc = 0.0f;
-#pragma unroll 8
-    for (int s = 0; s < p.splits; ++s) {
-        const float *rp = base + s * stride;
-        const float f = exp2f(rp[HD] - m);
-        l += f * rp[HD + 1];
-        acc += f * rp[d];
+    if (p.context_lens[seq] <= 0) return;
+    const int d = threadIdx.x % HD;
+    int q0 = seq;
+    bool have_q0 = !p.q_lens;
+    {
+        const int r = (int)blockIdx.z * RPW + (int)threadIdx.x / HD;
+        const int row = (int)blockIdx.y * 64 + r;
+        if (row >= rows_total) return;                  // uniform per wavefront (HD >= 64)
+        const float *base = p.part + ((((size_t)blockIdx.x * gridDim.y + blockIdx.y) * p.splits) * 64 + r) * (HD + 2);
+        const size_t stride = (size_t)64 * (HD + 2);
+        // one pass, 8 slices at a time (all their loads in flight together), rescaling the running
+        // sums whenever a batch raises the reference point
+        float m = -INFINITY, l = 0.0f, acc = 0.0f;
+        for (int s0 = 0; s0 < p.splits; s0 += 8) {
+            float ms[8], ls[8], os[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const float *rp = base + (size_t)min(s0 + u, p.splits - 1) * stride;
+                const bool in = s0 + u < p.splits;
+                ms[u] = in ? rp[HD] : -INFINITY;
+                ls[u] = in ? rp[HD + 1] : 0.0f;
+                os[u] = in ? rp[d] : 0.0f;
+            }
+            float mb = m;
+#pragma unroll
+            for (int u = 0; u < 8; ++u) mb = fmaxf(mb, ms[u]);
+            const float ref = mb == -INFINITY ? 0.0f : mb;
+            const float keep = exp2f(m - ref);            // m = -inf -> 0
+            l *= keep;
+            acc *= keep;
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const float f = exp2f(ms[u] - ref);
+                l += f * ls[u];
+                acc += f * os[u];
+            }
+            m = mb;
+        }
+        if (!have_q0) {
+            q0 = attn_first_token(p.q_lens, seq);
+            have_q0 = true;
+        }
+        const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+        const int tok = row / Gq, hq = row % Gq;
+        ((uint16_t *)p.out)[((size_t)(q0 + tok) * p.H + kvh * Gq + hq) * HD + d] = AttnT<T>::from_f32(acc * inv);
     }
-    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
-    const int tok = row / Gq, hq = row % Gq;
-    ((uint16_t *)p.out)[((size_t)(q0 + tok) * p.H + kvh * Gq + hq) * HD + d] = AttnT<T>::from_f32(acc * inv);
 }
 
 #ifndef ATTN_TARGET_WGS
