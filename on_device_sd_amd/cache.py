@@ -3,7 +3,11 @@
 ``evict`` / ``prefetch_async`` / ``complete_ready_transfers`` / ``get_cache_stats`` / ``reset_stats``
 / ``clear``, the same replacement-strategy protocol (``on_access``, ``on_insert``, ``on_evict``,
 ``select_victim(cached_experts, pinned_experts)``; ``demo/src/scheduling/cache_strategy.py``) and the
-same hit / miss accounting.
+same hit / miss accounting.  The bookkeeping methods (``get``, ``evict``, the victim loop,
+``prefetch_async``, ``complete_ready_transfers``, ``get_cache_stats``) restate the reference's
+bodies step by step, with its attribute names and statistics keys, because their observable
+behaviour -- what counts as a hit, when the strategy is told, which keys the statistics carry -- is
+the interface the engine and its tests rely on (``expert_cache.py:48-69, 125-151, 182-230``).
 
 What differs is the storage.  The reference keeps a dict of freshly allocated fp16 tensors per
 expert and frees them on eviction.  Here the cache owns a fixed pool of slots in HBM, each the
