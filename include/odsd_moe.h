@@ -241,6 +241,24 @@ size_t odsd_paged_attention_workspace_bytes(int32_t n_seqs, int32_t max_q_len, i
                                             int32_t num_kv_heads, int32_t head_dim, int32_t block_size,
                                             int32_t max_blocks);
 
+/* Causal attention of a prefill step: variable-length sequences packed one after the other, keys
+ * and values taken from the step's own k / v (no cache read).
+ *   q [total_q, num_heads, head_dim], k / v [total_k, num_kv_heads, head_dim], contiguous
+ *   cu_seqlens_q / cu_seqlens_k  int32 [n_seqs + 1]: row ranges of the sequences
+ *   query i of a sequence attends keys 0 .. i + (k_len - q_len) of it (the mask is aligned to
+ *   the bottom right corner when the lengths differ, as in flash-attn >= 2.1)
+ * max_seqlen_q / max_seqlen_k: upper bounds of the lengths; softmax_scale > 0; head_dim 64 or 128;
+ * workspace: odsd_varlen_attention_workspace_bytes(...) bytes.
+ * Stands in for the flash_attn_varlen_func call of Qwen3Attention.forward
+ * (demo/src/layers/attention.py:229-240; flash_attn itself is not part of the reference tree). */
+int     odsd_varlen_attention(const void *q, const void *k, const void *v, const int32_t *cu_seqlens_q,
+                              const int32_t *cu_seqlens_k, int32_t n_seqs, int32_t max_seqlen_q,
+                              int32_t max_seqlen_k, int32_t num_heads, int32_t num_kv_heads,
+                              int32_t head_dim, float softmax_scale, int32_t dtype, void *out,
+                              void *workspace, size_t workspace_bytes, void *stream);
+size_t odsd_varlen_attention_workspace_bytes(int32_t n_seqs, int32_t max_seqlen_q, int32_t max_seqlen_k,
+                                             int32_t num_heads, int32_t num_kv_heads, int32_t head_dim);
+
 /* The same call with every kernel timed, for measurement (no counterpart in the reference):
  * events = 2 * ODSD_N_KERNELS hipEvent_t handles created by the caller; the launch of kernel slot k
  * carries events[2k] and events[2k+1] as its start and stop events (hipExtLaunchKernel), so after

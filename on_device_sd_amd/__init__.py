@@ -12,7 +12,7 @@ from .placement import (ExpertActivation, LayerExpertActivations, build_layer_ac
                         build_prefill_placement)
 from .layers import W4MoELayer, W4MoELayerWithWeights, W4Operators
 from .cache import LRUStrategy, W4ExpertCache, cache_capacity
-from .kv import SequenceSlots, build_verify_context, paged_attention, store_kvcache
+from .kv import SequenceSlots, build_verify_context, paged_attention, store_kvcache, varlen_attention
 
 __all__ = [
     "AttentionOutput", "ExpertID", "ExpertPlacement", "LayerOutput", "MoEConfig", "RoutingResult",
@@ -21,5 +21,5 @@ __all__ = [
     "ExpertActivation", "LayerExpertActivations", "build_layer_activations", "build_prefill_placement",
     "W4MoELayer", "W4MoELayerWithWeights", "W4Operators",
     "LRUStrategy", "W4ExpertCache", "cache_capacity",
-    "SequenceSlots", "build_verify_context", "paged_attention", "store_kvcache",
+    "SequenceSlots", "build_verify_context", "paged_attention", "store_kvcache", "varlen_attention",
 ]

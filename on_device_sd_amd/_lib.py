@@ -59,6 +59,9 @@ SIGNATURES = {
     "odsd_paged_attention": (C.c_int, [_P, _P, _P, _P, _P, _P, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
                                        C.c_int32, C.c_int32, C.c_int64, C.c_float, C.c_int32, _P, _P, C.c_size_t, _P]),
     "odsd_paged_attention_workspace_bytes": (C.c_size_t, [C.c_int32] * 7),
+    "odsd_varlen_attention": (C.c_int, [_P, _P, _P, _P, _P] + [C.c_int32] * 6 + [C.c_float, C.c_int32, _P, _P,
+                                                                                C.c_size_t, _P]),
+    "odsd_varlen_attention_workspace_bytes": (C.c_size_t, [C.c_int32] * 6),
     "odsd_moe_forward_events": (C.c_int, [_SP, _P, _P, C.c_float, _P, _P, C.c_int32, _P, _P, _P, _P, _P,
                                           C.c_size_t, _P, _P, _P]),
     "odsd_moe_forward_static": (C.c_int, [_SP, _P, _P, C.c_float, _P, _P, C.c_int32, _P, _P, _P, _P, _P,

@@ -37,6 +37,9 @@ struct AttnParams {
     int n_seqs, H, KVH, max_blocks, block_size;
     int64_t num_slots;
     float scale_log2e;         // softmax scale * log2(e)
+    // variable-length mode (prefill): q / k / v rows of sequence s are q[cu_q[s] ..], k[cu_k[s] ..]
+    // (contiguous, no block table); both null in paged mode
+    const int32_t *cu_q, *cu_k;
     int splits;                // workgroups sharing one sequence's keys (blockIdx.z)
     float *part;               // splits > 1: partial results [seq, kvh, row group][split][64][HD + 2]
 };
@@ -97,8 +100,10 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int c = lane & 15, kq = lane >> 4;
     const int Gq = p.H / p.KVH;
-    const int L = p.context_lens[seq];
-    const int ql = p.q_lens ? p.q_lens[seq] : 1;
+    const bool varlen = p.cu_k != nullptr;
+    const int k_start = varlen ? p.cu_k[seq] : 0;
+    const int L = varlen ? p.cu_k[seq + 1] - k_start : p.context_lens[seq];
+    const int ql = varlen ? p.cu_q[seq + 1] - p.cu_q[seq] : (p.q_lens ? p.q_lens[seq] : 1);
     const int rows_total = ql * Gq;
     if (L <= 0 || ql <= 0 || (int)blockIdx.y * 64 >= rows_total) return;
     const int row0 = ((int)blockIdx.y * 4 + wave) * 16;
@@ -116,7 +121,8 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
     V8 qf[NJ];
     int q0 = seq;
     auto load_q = [&]() {
-        if (p.q_lens) q0 = attn_first_token(p.q_lens, seq);
+        if (varlen) q0 = p.cu_q[seq];
+        else if (p.q_lens) q0 = attn_first_token(p.q_lens, seq);
         const uint16_t *qp = (const uint16_t *)p.q + ((size_t)(q0 + tok) * p.H + kvh * Gq + hq) * HD + 8 * kq;
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
@@ -155,7 +161,7 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
     constexpr int NE = ALIGNED ? 1 : PIECES;            // table entries a tile needs per lane
     const int k_last = L - 1;
     const int bs = p.block_size;
-    auto entry_at = [&](int pos) -> int32_t { return bt[min(min(pos, k_last) / bs, p.max_blocks - 1)]; };
+    auto entry_at = [&](int pos) -> int32_t { return varlen ? 0 : bt[min(min(pos, k_last) / bs, p.max_blocks - 1)]; };
     auto request = [&](int k0, int32_t (&e)[NE]) {
         if constexpr (ALIGNED) {
             e[0] = entry_at(k0);
@@ -182,8 +188,8 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
             const int k0c = min(k0, k_last & ~31);
             const int blk = k0c / bs;
             const int32_t b = e[0];
-            const bool ok = b >= 0 && blk < p.max_blocks && ((int64_t)b + 1) * bs <= p.num_slots;
-            const int64_t slot0 = ok ? (int64_t)b * bs + (k0c - blk * bs) : 0;
+            const bool ok = varlen || (b >= 0 && blk < p.max_blocks && ((int64_t)b + 1) * bs <= p.num_slots);
+            const int64_t slot0 = varlen ? (int64_t)k_start + k0c : (ok ? (int64_t)b * bs + (k0c - blk * bs) : 0);
             const int lim = ok ? k_last - k0c : 0;
             const size_t base = (size_t)slot0 * D + kvh * HD;
             const uint16_t *kb = kc + base, *vb = vc + base;
@@ -223,7 +229,11 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
     };
 
     // this workgroup's slice of the 32-key tiles
-    const int all_tiles = (L + 31) / 32;
+    // (keys past the last one that any row of this workgroup attends are never visited: in a
+    // prefill the early row groups stop long before the end of the sequence)
+    const int last_tok = min(ql - 1, ((int)blockIdx.y * 64 + 63) / Gq);
+    const int k_end = min(L, L - ql + last_tok + 1);
+    const int all_tiles = (k_end + 31) / 32;
     const int per_split = (all_tiles + p.splits - 1) / p.splits;
     const int t_begin = min(all_tiles, (int)blockIdx.z * per_split);
     const int n_tiles = min(all_tiles, t_begin + per_split) - t_begin;
@@ -395,12 +405,14 @@ __global__ __launch_bounds__(256) void paged_attn_merge_kernel(const AttnParams 
     constexpr int RPW = 256 / HD;                       // rows per workgroup
     const int seq = blockIdx.x / p.KVH, kvh = blockIdx.x % p.KVH;
     const int Gq = p.H / p.KVH;
-    const int ql = p.q_lens ? p.q_lens[seq] : 1;
+    const bool varlen = p.cu_k != nullptr;
+    const int ql = varlen ? p.cu_q[seq + 1] - p.cu_q[seq] : (p.q_lens ? p.q_lens[seq] : 1);
     const int rows_total = ql * Gq;
-    if (p.context_lens[seq] <= 0) return;
+    if ((varlen ? p.cu_k[seq + 1] - p.cu_k[seq] : p.context_lens[seq]) <= 0) return;
     const int d = threadIdx.x % HD;
     int q0 = seq;
-    bool have_q0 = !p.q_lens;
+    bool have_q0 = !p.q_lens || varlen;
+    if (varlen) q0 = p.cu_q[seq];
     {
         const int r = (int)blockIdx.z * RPW + (int)threadIdx.x / HD;
         const int row = (int)blockIdx.y * 64 + r;
@@ -509,6 +521,66 @@ extern "C" int odsd_paged_attention(const void *q, const void *k_cache, const vo
     do {                                                                             \
         if (block_size % 32 == 0) paged_attn_kernel<T, HDV, true><<<grid, 256, 0, st>>>(p);  \
         else paged_attn_kernel<T, HDV, false><<<grid, 256, 0, st>>>(p);              \
+        if (p.splits > 1) paged_attn_merge_kernel<T, HDV><<<mgrid, 256, 0, st>>>(p); \
+    } while (0)
+    if (dtype == ODSD_DT_F16) {
+        if (head_dim == 128) ATTN_GO(half_t, 128);
+        else ATTN_GO(half_t, 64);
+    } else {
+        if (head_dim == 128) ATTN_GO(__bf16, 128);
+        else ATTN_GO(__bf16, 64);
+    }
+#undef ATTN_GO
+    ODSD_CHECK_LAUNCH();
+    return ODSD_OK;
+}
+
+// ---- variable-length (prefill) form ----------------------------------------------------------------
+extern "C" size_t odsd_varlen_attention_workspace_bytes(int32_t n_seqs, int32_t max_seqlen_q, int32_t max_seqlen_k,
+                                                        int32_t num_heads, int32_t num_kv_heads, int32_t head_dim) {
+    if (max_seqlen_k <= 0) return 0;
+    return odsd_paged_attention_workspace_bytes(n_seqs, max_seqlen_q, num_heads, num_kv_heads, head_dim, 32,
+                                                (max_seqlen_k + 31) / 32);
+}
+
+extern "C" int odsd_varlen_attention(const void *q, const void *k, const void *v, const int32_t *cu_seqlens_q,
+                                     const int32_t *cu_seqlens_k, int32_t n_seqs, int32_t max_seqlen_q,
+                                     int32_t max_seqlen_k, int32_t num_heads, int32_t num_kv_heads,
+                                     int32_t head_dim, float softmax_scale, int32_t dtype, void *out,
+                                     void *workspace, size_t workspace_bytes, void *stream) {
+    if (n_seqs < 0 || max_seqlen_q <= 0 || max_seqlen_k <= 0 || num_heads <= 0 || num_kv_heads <= 0 ||
+        num_heads % num_kv_heads || !(softmax_scale > 0.0f))
+        return ODSD_ERR_SHAPE;
+    if (head_dim != 64 && head_dim != 128) return ODSD_ERR_UNSUPPORTED;
+    if (dtype != ODSD_DT_BF16 && dtype != ODSD_DT_F16) return ODSD_ERR_DTYPE;
+    if (n_seqs == 0) return ODSD_OK;
+    if (!q || !k || !v || !cu_seqlens_q || !cu_seqlens_k || !out) return ODSD_ERR_NULL;
+    if (!odsd_aligned16(q) || !odsd_aligned16(k) || !odsd_aligned16(v)) return ODSD_ERR_ALIGN;
+    if ((int64_t)n_seqs * num_kv_heads > 0x7fffffffLL) return ODSD_ERR_SHAPE;
+    AttnParams p{};
+    p.q = q; p.k_cache = k; p.v_cache = v; p.out = out;
+    p.cu_q = cu_seqlens_q; p.cu_k = cu_seqlens_k;
+    p.n_seqs = n_seqs; p.H = num_heads; p.KVH = num_kv_heads;
+    p.block_size = 32; p.max_blocks = (max_seqlen_k + 31) / 32; p.num_slots = 0;
+    p.scale_log2e = softmax_scale * 1.4426950408889634f;
+    const int64_t rows = (int64_t)max_seqlen_q * (num_heads / num_kv_heads);
+    if ((rows + 63) / 64 > 65535) return ODSD_ERR_UNSUPPORTED;     // grid.y
+    const int rg = (int)((rows + 63) / 64);
+    p.splits = attn_splits(n_seqs, num_kv_heads, rg, p.max_blocks, 32);
+    if (p.splits > 1) {
+        const size_t need = odsd_varlen_attention_workspace_bytes(n_seqs, max_seqlen_q, max_seqlen_k, num_heads,
+                                                                  num_kv_heads, head_dim);
+        if (!workspace) return ODSD_ERR_NULL;
+        if (!odsd_aligned16(workspace)) return ODSD_ERR_ALIGN;
+        if (workspace_bytes < need) return ODSD_ERR_WORKSPACE;
+        p.part = (float *)workspace;
+    }
+    const dim3 grid((unsigned)(n_seqs * num_kv_heads), (unsigned)rg, (unsigned)p.splits);
+    const dim3 mgrid((unsigned)(n_seqs * num_kv_heads), (unsigned)rg, (unsigned)(64 / (256 / head_dim)));
+    hipStream_t st = (hipStream_t)stream;
+#define ATTN_GO(T, HDV)                                                              \
+    do {                                                                             \
+        paged_attn_kernel<T, HDV, true><<<grid, 256, 0, st>>>(p);                    \
         if (p.splits > 1) paged_attn_merge_kernel<T, HDV><<<mgrid, 256, 0, st>>>(p); \
     } while (0)
     if (dtype == ODSD_DT_F16) {

@@ -97,6 +97,44 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     return out
 
 
+def varlen_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens_q: torch.Tensor,
+                     cu_seqlens_k: torch.Tensor, max_seqlen_q: int, max_seqlen_k: int,
+                     softmax_scale: Optional[float] = None, causal: bool = True) -> torch.Tensor:
+    """The ``flash_attn_varlen_func`` call of a prefill step (``attention.py:229-240``), same
+    arguments: q [total_q, num_heads, head_dim], k / v [total_k, num_kv_heads, head_dim] packed
+    sequence after sequence, ``cu_seqlens_*`` int32 [n_seqs + 1].  Causal only (what the reference
+    asks for); with unequal lengths the mask is aligned to the bottom right corner."""
+    if not causal:
+        raise NotImplementedError("the reference's prefill attention is causal; only that form is built")
+    if not (q.is_cuda and k.is_cuda and v.is_cuda):
+        raise RuntimeError("attention runs on the GPU only (there is no CPU fallback)")
+    total_q, num_heads, head_dim = q.shape
+    num_kv_heads = k.shape[1]
+    assert q.is_contiguous() and k.is_contiguous() and v.is_contiguous()
+    assert k.shape == v.shape and k.shape[2] == head_dim and q.dtype == k.dtype == v.dtype
+    dt = {torch.bfloat16: _lib.DT_BF16, torch.float16: _lib.DT_F16}.get(q.dtype)
+    if dt is None:
+        raise TypeError("attention takes bfloat16 or float16")
+    cq = cu_seqlens_q.to(torch.int32).contiguous()
+    ck = cu_seqlens_k.to(torch.int32).contiguous()
+    n_seqs = cq.numel() - 1
+    out = torch.empty_like(q)
+    if n_seqs <= 0 or total_q == 0:
+        return out
+    scale = head_dim ** -0.5 if softmax_scale is None else softmax_scale
+    lib = _lib.load()
+    nbytes = lib.odsd_varlen_attention_workspace_bytes(n_seqs, max_seqlen_q, max_seqlen_k, num_heads, num_kv_heads,
+                                                       head_dim)
+    if nbytes == 0:
+        raise _lib.OdsdError("attention: unsupported shape (head_dim 64 or 128, heads a multiple of KV heads)")
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+    _lib.check(lib.odsd_varlen_attention(q.data_ptr(), k.data_ptr(), v.data_ptr(), cq.data_ptr(), ck.data_ptr(), n_seqs,
+                                         max_seqlen_q, max_seqlen_k, num_heads, num_kv_heads, head_dim, scale, dt,
+                                         out.data_ptr(), ws.data_ptr(), nbytes,
+                                         torch.cuda.current_stream().cuda_stream), "odsd_varlen_attention")
+    return out
+
+
 @dataclass
 class SequenceSlots:
     """What the slot arithmetic needs of a sequence (``SequenceState``, paged_kv_cache.py:127-207)."""

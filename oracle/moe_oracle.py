@@ -482,3 +482,35 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                                            is_causal=False, scale=scale)
         outs.append(o.squeeze(0).transpose(0, 1))
     return torch.cat(outs, dim=0)
+
+
+def varlen_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_q, cu_k, scale: float) -> torch.Tensor:
+    """The prefill attention of Qwen3Attention.forward (demo/src/layers/attention.py:229-240):
+    flash_attn_varlen_func(q, k, v, cu_seqlens_q, cu_seqlens_k, ..., causal=True) in fp32.
+    flash_attn is a third-party package that the reference neither vendors nor pins; its
+    published semantics are restated: the sequences are packed one after the other, KV heads are
+    shared by consecutive groups of query heads, softmax(q k^T * scale) v per sequence, and with
+    causal=True query i sees keys j <= i + (k_len - q_len) (mask aligned to the bottom right
+    corner, flash-attn >= 2.1; identical to the usual lower triangle when the lengths agree, which
+    is the reference's prefill).  q [total_q, H, HD]; k, v [total_k, KVH, HD]."""
+    total_q, H, HD = q.shape
+    KVH = k.shape[1]
+    qf, kf, vf = q.to(torch.float32), k.to(torch.float32), v.to(torch.float32)
+    cu_q = np.asarray(cu_q).tolist()
+    cu_k = np.asarray(cu_k).tolist()
+    outs = []
+    for s in range(len(cu_q) - 1):
+        qs = qf[cu_q[s]:cu_q[s + 1]]
+        ks = kf[cu_k[s]:cu_k[s + 1]].repeat_interleave(H // KVH, dim=1)
+        vs = vf[cu_k[s]:cu_k[s + 1]].repeat_interleave(H // KVH, dim=1)
+        ql, kl = qs.shape[0], ks.shape[0]
+        if ql == 0:
+            continue
+        scores = torch.einsum("qhd,khd->hqk", qs, ks) * scale
+        allowed = torch.arange(kl)[None, :] <= (torch.arange(ql)[:, None] + (kl - ql))
+        scores = scores.masked_fill(~allowed[None], float("-inf"))
+        probs = torch.softmax(scores, dim=-1)
+        probs = torch.nan_to_num(probs, nan=0.0)       # a query with no visible key (k_len < q_len) gives zeros
+        outs.append(torch.einsum("hqk,khd->qhd", probs, vs))
+    return torch.cat(outs, dim=0) if outs else qf.new_zeros((0, H, HD))
+

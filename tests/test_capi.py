@@ -100,6 +100,16 @@ def test_argument_checks_need_no_gpu():
     assert lib.odsd_paged_attention_workspace_bytes(2, 8, 32, 4, 96, 256, 16) == 0
     # many sequences: one workgroup per (sequence, KV head) walks all its keys, no partial results
     assert lib.odsd_paged_attention_workspace_bytes(512, 1, 32, 4, 128, 256, 16) == 256
+    # variable-length (prefill) attention: q, k, v, cu_q, cu_k, n_seqs, max_q, max_k, H, KVH, HD, scale, dtype,
+    # out, workspace, workspace_bytes, stream
+    var = lambda *a: lib.odsd_varlen_attention(*a)
+    assert var(P, P, P, P, P, 2, 64, 64, 32, 4, 128, 0.1, _lib.DT_BF16, None, None, 0, None) == 1
+    assert var(P, P, P, P, P, 2, 64, 64, 32, 4, 128, 0.0, _lib.DT_BF16, P, None, 0, None) == 2
+    assert var(P, P, P, P, P, 2, 64, 64, 32, 4, 80, 0.1, _lib.DT_BF16, P, None, 0, None) == 3
+    assert var(P, P, P, P, P, 2, 64, 64, 32, 4, 128, 0.1, _lib.DT_F32, P, None, 0, None) == 7
+    assert var(None, None, None, None, None, 0, 64, 64, 32, 4, 128, 0.1, _lib.DT_BF16, None, None, 0, None) == 0
+    assert lib.odsd_varlen_attention_workspace_bytes(2, 64, 64, 32, 4, 128) == 256       # short: no key slicing
+    assert lib.odsd_varlen_attention_workspace_bytes(1, 8, 8192, 32, 4, 128) > 256
     empty = _lib.MoeShape(0, 256, 8, 2, 256, 1, _lib.DT_BF16, 0)       # T == 0 is a no-op
     assert lib.odsd_dispatch(C.byref(empty), 1 << 20, 1 << 20, 1 << 20, 1 << 20, 1 << 20, 1 << 20, None) == 0
 

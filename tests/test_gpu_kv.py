@@ -114,3 +114,30 @@ def test_paged_attention_vs_oracle(dev, dtype, H, KVH, HD, bs, seqs):
     out2 = odsd.paged_attention(q.to(dev), kc.to(dev), vc.to(dev), ctx, KVH, bs,
                                 max_q_len=None if decode else int(qlens.max()))
     assert torch.equal(out, out2)
+
+
+VARLEN_CASES = [
+    # dtype, H, KVH, HD, (q_len, k_len) per sequence
+    (torch.bfloat16, 32, 4, 128, [(300, 300), (1, 1), (77, 77)]),            # Qwen3-30B-A3B heads, ragged prefill batch
+    (torch.float16, 8, 8, 64, [(130, 130), (64, 64)]),                      # no grouping, head_dim 64
+    (torch.bfloat16, 16, 2, 128, [(40, 200), (5, 5), (64, 65)]),            # queries on top of earlier keys (chunked prefill)
+    (torch.bfloat16, 32, 4, 128, [(1500, 1500)]),                           # one long sequence: many row groups, early key cut-off
+]
+
+
+@pytest.mark.parametrize("dtype,H,KVH,HD,seqs", VARLEN_CASES)
+def test_varlen_attention_vs_oracle(dev, dtype, H, KVH, HD, seqs):
+    print("varlen attention", dtype, H, KVH, HD, seqs, flush=True)
+    import on_device_sd_amd as odsd
+    g = torch.Generator().manual_seed(H + HD + len(seqs))
+    cu_q = np.concatenate([[0], np.cumsum([a for a, _ in seqs])]).astype(np.int32)
+    cu_k = np.concatenate([[0], np.cumsum([b for _, b in seqs])]).astype(np.int32)
+    q = torch.randn(int(cu_q[-1]), H, HD, generator=g).to(dtype)
+    k = torch.randn(int(cu_k[-1]), KVH, HD, generator=g).to(dtype)
+    v = torch.randn(int(cu_k[-1]), KVH, HD, generator=g).to(dtype)
+    out = odsd.varlen_attention(q.to(dev), k.to(dev), v.to(dev), torch.from_numpy(cu_q).to(dev), torch.from_numpy(cu_k).to(dev),
+                                max(a for a, _ in seqs), max(b for _, b in seqs), softmax_scale=HD ** -0.5)
+    ref = orc.varlen_attention(q, k, v, cu_q, cu_k, HD ** -0.5)
+    err = (out.float().cpu() - ref).abs()
+    print(f"  max-abs error {err.max().item():.3e} (max|ref| {ref.abs().max().item():.2f})", flush=True)
+    assert err.max().item() <= 2e-2 and err.mean().item() <= 2e-3

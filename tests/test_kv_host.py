@@ -80,3 +80,49 @@ def test_oracle_paged_attention_against_plain_softmax():
     dec = orc.paged_attention(q[:2], kc, vc, tables, lens, None, KVH, bs, 0.3)
     one = orc.paged_attention(q[:2], kc, vc, tables, lens, [1, 1], KVH, bs, 0.3)
     assert torch.equal(dec, one)
+
+
+def test_oracle_varlen_attention_pins():
+    """The prefill attention restatement against (a) the library's own causal SDPA per sequence
+    when the lengths agree (the reference's prefill), (b) a scalar loop when keys outnumber
+    queries (bottom-right aligned mask), (c) the paged form: a prefill whose K / V were stored in
+    the cache first must give the same result through the block tables."""
+    import torch.nn.functional as F
+    g = torch.Generator().manual_seed(1)
+    H, KVH, HD = 4, 2, 8
+    lens = [5, 1, 9]
+    cu = np.concatenate([[0], np.cumsum(lens)])
+    q = torch.randn(cu[-1], H, HD, generator=g)
+    k = torch.randn(cu[-1], KVH, HD, generator=g)
+    v = torch.randn(cu[-1], KVH, HD, generator=g)
+    out = orc.varlen_attention(q, k, v, cu, cu, 0.4)
+    for s, L in enumerate(lens):
+        sl = slice(cu[s], cu[s + 1])
+        ks = k[sl].repeat_interleave(H // KVH, dim=1)
+        vs = v[sl].repeat_interleave(H // KVH, dim=1)
+        ref = F.scaled_dot_product_attention(q[sl].transpose(0, 1)[None], ks.transpose(0, 1)[None], vs.transpose(0, 1)[None],
+                                             is_causal=True, scale=0.4)[0].transpose(0, 1)
+        assert torch.allclose(out[sl], ref, atol=1e-5)
+    # (b) 2 queries on 6 keys: query j sees keys 0 .. j + 4
+    q2, k2, v2 = q[:2], k[:6], v[:6]
+    o2 = orc.varlen_attention(q2, k2, v2, [0, 2], [0, 6], 0.4)
+    for j in range(2):
+        for h in range(H):
+            kvh = h // (H // KVH)
+            sc = [float(q2[j, h] @ k2[p, kvh]) * 0.4 for p in range(j + 5)]
+            w = np.exp(np.array(sc) - max(sc))
+            ref = sum(wi * v2[p, kvh] for p, wi in enumerate(w)) / w.sum()
+            assert torch.allclose(o2[j, h], ref.to(torch.float32), atol=1e-5)
+    # (c) the same prefill through a cache with 4-token blocks in scrambled order
+    bs = 4
+    tables, kc, vc, nxt = [], torch.zeros(8 * bs, KVH * HD), torch.zeros(8 * bs, KVH * HD), [5, 2, 7, 0, 3, 6, 1, 4]
+    at = 0
+    for s, L in enumerate(lens):
+        nb = -(-L // bs)
+        tab = nxt[at:at + nb]; at += nb
+        tables.append(tab + [-1] * (3 - nb))
+        for p in range(L):
+            kc[tab[p // bs] * bs + p % bs] = k[cu[s] + p].reshape(-1)
+            vc[tab[p // bs] * bs + p % bs] = v[cu[s] + p].reshape(-1)
+    paged = orc.paged_attention(q, kc, vc, tables, lens, lens, KVH, bs, 0.4)
+    assert torch.allclose(paged, out, atol=1e-5)
