@@ -141,3 +141,58 @@ def test_varlen_attention_vs_oracle(dev, dtype, H, KVH, HD, seqs):
     err = (out.float().cpu() - ref).abs()
     print(f"  max-abs error {err.max().item():.3e} (max|ref| {ref.abs().max().item():.2f})", flush=True)
     assert err.max().item() <= 2e-2 and err.mean().item() <= 2e-3
+
+
+def test_paged_and_varlen_attention_random_shapes(dev):
+    """Seeded random shapes: query-head group sizes that do not divide 64, block sizes 1..64 (both
+    table paths), contexts shorter than a key tile, contexts long enough for several key slices,
+    query lengths from 1 to the whole context; every case through the paged entry point and, with
+    the same rows packed, through the variable-length one."""
+    import on_device_sd_amd as odsd
+    rng = np.random.default_rng(2024)
+    worst = 0.0
+    for case in range(24):
+        HD = int(rng.choice([64, 128]))
+        KVH = int(rng.choice([1, 2, 4]))
+        Gq = int(rng.choice([1, 2, 3, 6, 8, 16]))
+        H = KVH * Gq
+        bs = int(rng.choice([1, 3, 16, 32, 64]))
+        dtype = torch.bfloat16 if case % 2 else torch.float16
+        n_seqs = int(rng.integers(1, 5))
+        seqs = []
+        for _ in range(n_seqs):
+            L = int(rng.choice([rng.integers(1, 40), rng.integers(40, 400), rng.integers(1000, 2600)]))
+            ql = int(rng.choice([1, min(L, 5), min(L, int(rng.integers(1, 70))), L if L < 300 else 1]))
+            seqs.append((L, ql))
+        print("random attention case", case, dtype, H, KVH, HD, bs, seqs, flush=True)
+        g = torch.Generator().manual_seed(case)
+        nbs = [-(-L // bs) for L, _ in seqs]
+        perm = torch.randperm(sum(nbs) + 2, generator=g).tolist()
+        tables, at = [], 0
+        for nb in nbs:
+            tables.append(perm[at:at + nb]); at += nb
+        mb = max(nbs)
+        bt = torch.tensor([t + [-1] * (mb - len(t)) for t in tables], dtype=torch.int32)
+        D = KVH * HD
+        kc = torch.randn((sum(nbs) + 2) * bs, D, generator=g).to(dtype)
+        vc = torch.randn((sum(nbs) + 2) * bs, D, generator=g).to(dtype)
+        q = torch.randn(sum(ql for _, ql in seqs), H, HD, generator=g).to(dtype)
+        lens = [L for L, _ in seqs]
+        qls = [ql for _, ql in seqs]
+        ctx = {"block_tables": bt.to(dev), "context_lens": torch.tensor(lens, dtype=torch.int32, device=dev),
+               "verify_query_lens": torch.tensor(qls, dtype=torch.int32, device=dev)}
+        out = odsd.paged_attention(q.to(dev), kc.to(dev), vc.to(dev), ctx, KVH, bs, max_q_len=max(qls))
+        ref = orc.paged_attention(q, kc, vc, bt.tolist(), lens, qls, KVH, bs, HD ** -0.5)
+        err = (out.float().cpu() - ref).abs()
+        assert err.max().item() <= 2e-2 and err.mean().item() <= 2e-3, (case, err.max().item())
+        worst = max(worst, err.max().item())
+        # the same keys packed sequence after sequence
+        rows = [torch.tensor([tables[i][p // bs] * bs + p % bs for p in range(L)]) for i, L in enumerate(lens)]
+        kp = torch.cat([kc[r] for r in rows]).view(-1, KVH, HD).contiguous()
+        vp = torch.cat([vc[r] for r in rows]).view(-1, KVH, HD).contiguous()
+        cu_q = torch.tensor([0] + list(np.cumsum(qls)), dtype=torch.int32)
+        cu_k = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+        out_v = odsd.varlen_attention(q.to(dev), kp.to(dev), vp.to(dev), cu_q.to(dev), cu_k.to(dev), max(qls), max(lens))
+        err_v = (out_v.float().cpu() - ref).abs()
+        assert err_v.max().item() <= 2e-2 and err_v.mean().item() <= 2e-3, (case, err_v.max().item())
+    print(f"  worst max-abs error {worst:.3e}", flush=True)
