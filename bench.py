@@ -326,6 +326,7 @@ def bench_attention(dev, steps, warmup, with_cpu):
     attn_ms = timed(g_attn.replay)
     kv_bytes = 2 * n_seqs * L * KVH * HD * 2 + 2 * q.numel() * 2
     ach = kv_bytes / (attn_ms * 1e-3) / 1e9
+    traffic, traffic_commit = _traffic(name)
     n_tok = n_seqs * ql
     res = {
         "workload": name, "kind": "kv-cache store + paged causal attention (one layer of a verify step)",
@@ -333,9 +334,11 @@ def bench_attention(dev, steps, warmup, with_cpu):
         "head_dim": HD, "block_size": bs, "tokens_per_s": round(n_tok / (graph_ms * 1e-3), 1),
         "ms_per_step": round(graph_ms, 5), "ms_per_step_eager_python": round(eager_ms, 5),
         "roofline": {"bound": "hbm", "kernel": "paged_attn_kernel + paged_attn_merge_kernel", "achieved": round(ach, 1),
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": traffic,
                      "algorithmic_bytes": kv_bytes, "kernel_ms": round(attn_ms, 5)},
     }
+    if traffic_commit:
+        res["roofline"]["traffic_measured_at_commit"] = traffic_commit
     if with_cpu:
         # the oracle's restatement of the reference's fallback attention on a sample of the sequences
         from oracle import moe_oracle as oracle
