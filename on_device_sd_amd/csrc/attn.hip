@@ -1,26 +1,34 @@
-// Causal attention of a decode / verify step over the paged KV cache (gfx950).
+// Causal attention over cached or packed keys (gfx950): the decode / verify step over the paged KV
+// cache, and the prefill step over the step's own variable-length sequences.
 //
-// One workgroup per (sequence, KV head, group of 64 query rows, slice of the keys); a query row is one (token, query
-// head) pair of the KV head's group, so with grouped-query attention a verify step of 8 tokens and
-// 8 query heads per KV head fills the 64 rows.  Each of the 4 wavefronts owns 16 rows and walks
-// the sequence's cached keys 32 at a time:
-//   * S^T = K Q^T on the matrix cores (v_mfma_f32_16x16x32, keys as the A operand straight from
-//     the cache rows, the wavefront's Q rows as the B operand held in registers), which leaves
-//     the scores of one query row in the 4 lanes that share lane % 16 -- the layout the P operand
-//     of the second product needs, so the probabilities never move between lanes;
-//   * online softmax in fp32 (running maximum and sum per row, exp2 with the scale folded in);
-//   * O += P V with V^T as the B operand: the 32 x head_dim tile of V is transposed through LDS
-//     once per workgroup (double buffered, one barrier per tile) and shared by the wavefronts.
+// One workgroup per (sequence, KV head, group of 64 query rows, slice of the keys); a query row is
+// one (token, query head) pair of the KV head's group, so with grouped-query attention a verify
+// step of 8 tokens and 8 query heads per KV head fills the 64 rows.  Each of the 4 wavefronts owns
+// 16 rows; the workgroup walks its keys 32 at a time:
+//   * the tile's K and V rows are fetched once per workgroup (two tiles ahead, into registers) and
+//     put into LDS one tile ahead: K as stored, V transposed; all wavefronts read their operands
+//     from there (double buffered, one barrier per tile);
+//   * S^T = K Q^T on the matrix cores (v_mfma_f32_16x16x32, keys as the A operand, the
+//     wavefront's Q rows as the B operand held in registers), which leaves the scores of one
+//     query row in the 4 lanes that share lane % 16 -- the layout the P operand of the second
+//     product needs, so the probabilities never move between lanes;
+//   * softmax in fp32 in the exp2 domain with the scale folded in; a row's reference point (the
+//     value subtracted before exp2) follows its running maximum lazily, and the sum of the
+//     probabilities stays a per-lane partial sum until the end, so most tiles exchange nothing
+//     between lanes;
+//   * O += P V with V^T as the B operand.
 // A verify step has few (sequence, KV head) pairs and long key lists, so the keys of one sequence
-// are cut into `splits` slices handled by different workgroups; each leaves its running maximum,
+// are cut into `splits` slices handled by different workgroups; each leaves its reference point,
 // sum and unnormalised output, and a small second kernel merges the slices of a row (the usual
 // rescaling by exp2(m_slice - m_all)), in slice order.
-// The cache is addressed through the sequence's block table exactly as the reference gathers it:
-// position p lives in slot block_table[p / block_size] * block_size + p % block_size.
+// Paged form: the cache is addressed through the sequence's block table exactly as the reference
+// gathers it: position p lives in slot block_table[p / block_size] * block_size + p % block_size.
+// Packed form: the keys of sequence s are rows cu_seqlens_k[s] .. of k / v.
 //
 // Replaces Qwen3Attention._fallback_decode_attention (demo/src/layers/attention.py:290-352: gather
 // of the cached K/V by slot, repeat_interleave for GQA, causal mask with offset k_len - q_len,
-// scaled_dot_product_attention) and the flash_attn_with_kvcache call it stands in for (:252-272).
+// scaled_dot_product_attention), the flash_attn_with_kvcache call it stands in for (:252-272) and
+// the flash_attn_varlen_func call of the prefill branch (:229-240).
 #include "common.h"
 #include <type_traits>
 
