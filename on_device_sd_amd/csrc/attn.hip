@@ -408,7 +408,7 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
 // order. One workgroup per (sequence, KV head, row group, 256 / HD rows): a thread owns one output
 // element and walks the slices, neighbouring threads reading neighbouring floats.  (More rows per
 // workgroup, taken in turn, measured slower: each turn is one more exposed load latency.)
-template <typename T, int HD>
+template <typename T, int HD, int SB>
 __global__ __launch_bounds__(256) void paged_attn_merge_kernel(const AttnParams p) {
     constexpr int RPW = 256 / HD;                       // rows per workgroup
     const int seq = blockIdx.x / p.KVH, kvh = blockIdx.x % p.KVH;
@@ -427,28 +427,36 @@ __global__ __launch_bounds__(256) void paged_attn_merge_kernel(const AttnParams 
         if (row >= rows_total) return;                  // uniform per wavefront (HD >= 64)
         const float *base = p.part + ((((size_t)blockIdx.x * gridDim.y + blockIdx.y) * p.splits) * 64 + r) * (HD + 2);
         const size_t stride = (size_t)64 * (HD + 2);
-        // one pass, 8 slices at a time (all their loads in flight together), rescaling the running
+        // one pass, SB slices at a time (all their loads in flight together; SB = 4 when there are no
+        // more than 4 slices, so that none is fetched twice), rescaling the running
         // sums whenever a batch raises the reference point
         float m = -INFINITY, l = 0.0f, acc = 0.0f;
-        for (int s0 = 0; s0 < p.splits; s0 += 8) {
-            float ms[8], ls[8], os[8];
+        for (int s0 = 0; s0 < p.splits; s0 += SB) {
+            float ms[SB], ls[SB], os[SB];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
+            for (int u = 0; u < SB; ++u) {
+                // (every load unconditional, on a clamped slice: loads under a branch serialise)
                 const float *rp = base + (size_t)min(s0 + u, p.splits - 1) * stride;
-                const bool in = s0 + u < p.splits;
-                ms[u] = in ? rp[HD] : -INFINITY;
-                ls[u] = in ? rp[HD + 1] : 0.0f;
-                os[u] = in ? rp[d] : 0.0f;
+                ms[u] = rp[HD];
+                ls[u] = rp[HD + 1];
+                os[u] = rp[d];
+            }
+#pragma unroll
+            for (int u = 0; u < SB; ++u) {
+                if (s0 + u >= p.splits) {
+                    ms[u] = -INFINITY;
+                    ls[u] = os[u] = 0.0f;
+                }
             }
             float mb = m;
 #pragma unroll
-            for (int u = 0; u < 8; ++u) mb = fmaxf(mb, ms[u]);
+            for (int u = 0; u < SB; ++u) mb = fmaxf(mb, ms[u]);
             const float ref = mb == -INFINITY ? 0.0f : mb;
             const float keep = exp2f(m - ref);            // m = -inf -> 0
             l *= keep;
             acc *= keep;
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
+            for (int u = 0; u < SB; ++u) {
                 const float f = exp2f(ms[u] - ref);
                 l += f * ls[u];
                 acc += f * os[u];
@@ -529,7 +537,8 @@ extern "C" int odsd_paged_attention(const void *q, const void *k_cache, const vo
     do {                                                                             \
         if (block_size % 32 == 0) paged_attn_kernel<T, HDV, true><<<grid, 256, 0, st>>>(p);  \
         else paged_attn_kernel<T, HDV, false><<<grid, 256, 0, st>>>(p);              \
-        if (p.splits > 1) paged_attn_merge_kernel<T, HDV><<<mgrid, 256, 0, st>>>(p); \
+        if (p.splits > 4) paged_attn_merge_kernel<T, HDV, 8><<<mgrid, 256, 0, st>>>(p);      \
+        else if (p.splits > 1) paged_attn_merge_kernel<T, HDV, 4><<<mgrid, 256, 0, st>>>(p); \
     } while (0)
     if (dtype == ODSD_DT_F16) {
         if (head_dim == 128) ATTN_GO(half_t, 128);
@@ -589,7 +598,8 @@ extern "C" int odsd_varlen_attention(const void *q, const void *k, const void *v
 #define ATTN_GO(T, HDV)                                                              \
     do {                                                                             \
         paged_attn_kernel<T, HDV, true><<<grid, 256, 0, st>>>(p);                    \
-        if (p.splits > 1) paged_attn_merge_kernel<T, HDV><<<mgrid, 256, 0, st>>>(p); \
+        if (p.splits > 4) paged_attn_merge_kernel<T, HDV, 8><<<mgrid, 256, 0, st>>>(p);      \
+        else if (p.splits > 1) paged_attn_merge_kernel<T, HDV, 4><<<mgrid, 256, 0, st>>>(p); \
     } while (0)
     if (dtype == ODSD_DT_F16) {
         if (head_dim == 128) ATTN_GO(half_t, 128);
