@@ -46,7 +46,8 @@
 extern "C" {
 #endif
 
-#define ODSD_VERSION 100
+/* 110: events / static forms of the whole block, KV store, paged and packed attention added (100: the MoE block) */
+#define ODSD_VERSION 110
 
 typedef enum odsd_status {
     ODSD_OK = 0,
