@@ -170,8 +170,8 @@ int odsd_experts_w4(const odsd_moe_shape *s, const void *x_f16, const uint64_t *
  * callers that keep h / y themselves or time the stages:
  *   h_f16 fp16 [P, I] in slot order; y: a buffer of odsd_w4_down_splits(s)*P*H*4 bytes that
  *   odsd_w4_down fills and odsd_combine reads -- float [splits][P][H] partial sums over slices
- *   of I, which odsd_combine adds in slice order, or, at prefill shapes (splits == 1, more than
- *   42 rows per expert on average), fp16 [P][H].
+ *   of I, which odsd_combine adds in slice order, or, when the reduction is not split
+ *   (splits == 1), fp16 [P][H].
  * They stand in for the three F.linear calls of mlp.py:227-230 (gate/up fused with
  * SiLU*mul, then down) and the indexed "+=" of qwen3_runner.py:363. */
 int     odsd_w4_gate_up_silu(const odsd_moe_shape *s, const void *x_f16, const uint64_t *table,

@@ -343,7 +343,13 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
                     for (int i = 0; i < NB; ++i) {
                         if (blk_ok[i]) {
                             const int n = (blk0 + i) * 16 + kq * 4;
-                            *(float4_t *)(p.y + ((size_t)ks * p.P + slot) * p.ldo + n) = acc[i][m];
+                            if (p.y_f16) {
+                                const float4_t v = acc[i][m];
+                                *(half4_t *)((half_t *)p.y + slot * p.ldo + n) =
+                                    half4_t{f32_to_f16_sat(v.x), f32_to_f16_sat(v.y), f32_to_f16_sat(v.z), f32_to_f16_sat(v.w)};
+                            } else {
+                                *(float4_t *)(p.y + ((size_t)ks * p.P + slot) * p.ldo + n) = acc[i][m];
+                            }
                         }
                     }
                 }
@@ -476,7 +482,7 @@ struct ExpertsPlan {
     int KS;          // split of the down projection's reduction dimension across workgroups
     int PS_gu, PS_dn;  // prefill tile kernel: workgroups sharing the row passes of one tile
     int tile;        // MB == 8: the 256 x 256 tile kernel instead of the streaming kernel
-    int y_f16;       // down-projection outputs kept as fp16 (prefill tile kernel) instead of fp32 partials
+    int y_f16;       // down-projection outputs kept as fp16 (unsplit reduction) instead of fp32 partials
     size_t h_bytes, y_bytes;
 };
 
@@ -537,9 +543,11 @@ static ExpertsPlan experts_plan(const odsd_moe_shape *s) {
     }
     // every split must own at least one group
     while (p.KS > 1 && ((G_dn + p.KS - 1) / p.KS) * (p.KS - 1) >= G_dn) p.KS--;
-    // At prefill shapes the fp32 partials would be 0.5 GB written and read back per layer; fp16
-    // still carries 3 more bits than the bf16 the reference keeps its expert outputs in.
-    p.y_f16 = p.tile && p.KS == 1;
+    // Without a split of the reduction the down projection's outputs are complete sums: they are
+    // stored as fp16 (3 more bits than the bf16 the reference keeps its expert outputs in), half the
+    // bytes to write and to read back in the combine (at prefill shapes fp32 would be 0.5 GB per
+    // layer each way).  Split reductions leave fp32 partial sums, added in order by the combine.
+    p.y_f16 = p.KS == 1;
     p.h_bytes = odsd_round_up((size_t)(P > 0 ? P : 1) * s->I * sizeof(half_t), 256);
     p.y_bytes = odsd_round_up((size_t)p.KS * (size_t)(P > 0 ? P : 1) * s->H * sizeof(float), 256);
     return p;
@@ -582,6 +590,7 @@ template <int MODE> void odsd_launch_gemm_prefill(GemmParams &gp, hipStream_t st
 template <int MODE>
 static void launch_gemm_plan(const ExpertsPlan &pl, GemmParams &gp, hipStream_t st) {
     const int wk = MODE == 0 ? pl.WK_gu : pl.WK_dn;
+    gp.y_f16 = pl.y_f16;
     if (pl.MB == 1) {
         if (wk == 4) launch_gemm<4, 1, MODE, 2, 2, 4, true, 2>(gp, st);
         else if (wk == 2) launch_gemm<4, 1, MODE, 3, 2, 2, true, 2>(gp, st);
@@ -593,7 +602,6 @@ static void launch_gemm_plan(const ExpertsPlan &pl, GemmParams &gp, hipStream_t 
         if (pl.NB == 2) launch_gemm<2, 4, MODE, 2, 2, 1, false, 4>(gp, st);
         else launch_gemm<4, 4, MODE, 2, 2, 1, false, 2>(gp, st);
     } else if (pl.tile) {
-        gp.y_f16 = pl.y_f16;
         odsd_launch_gemm_prefill<MODE>(gp, st);
     } else {
         launch_gemm<2, 8, MODE, 2, 2, 1, false, 2>(gp, st);
