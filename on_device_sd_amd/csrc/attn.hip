@@ -492,7 +492,9 @@ extern "C" size_t odsd_paged_attention_workspace_bytes(int32_t n_seqs, int32_t m
     if (n_seqs <= 0 || max_q_len <= 0 || num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads ||
         block_size <= 0 || max_blocks <= 0 || (head_dim != 64 && head_dim != 128))
         return 0;
-    const int rg = (max_q_len * (num_heads / num_kv_heads) + 63) / 64;
+    const int64_t rows = (int64_t)max_q_len * (num_heads / num_kv_heads);
+    if ((rows + 63) / 64 > 65535) return 0;
+    const int rg = (int)((rows + 63) / 64);
     const int splits = attn_splits(n_seqs, num_kv_heads, rg, max_blocks, block_size);
     if (splits == 1) return 256;
     return odsd_round_up((size_t)n_seqs * num_kv_heads * rg * splits * 64 * (head_dim + 2) * sizeof(float), 256);
@@ -520,7 +522,9 @@ extern "C" int odsd_paged_attention(const void *q, const void *k_cache, const vo
     p.n_seqs = n_seqs; p.H = num_heads; p.KVH = num_kv_heads; p.max_blocks = max_blocks;
     p.block_size = block_size; p.num_slots = num_slots;
     p.scale_log2e = softmax_scale * 1.4426950408889634f;
-    const int rg = (max_q_len * (num_heads / num_kv_heads) + 63) / 64;
+    const int64_t rows = (int64_t)max_q_len * (num_heads / num_kv_heads);
+    if ((rows + 63) / 64 > 65535) return ODSD_ERR_UNSUPPORTED;     // grid.y
+    const int rg = (int)((rows + 63) / 64);
     p.splits = attn_splits(n_seqs, num_kv_heads, rg, max_blocks, block_size);
     if (p.splits > 1) {
         const size_t need = odsd_paged_attention_workspace_bytes(n_seqs, max_q_len, num_heads, num_kv_heads,

@@ -98,6 +98,9 @@ def test_argument_checks_need_no_gpu():
     assert att(P, P, P, P, P, None, 2, 8, 32, 4, 128, 256, 16, 8192, 0.1, _lib.DT_BF16, P, None, 0, None) == 1
     assert att(P, P, P, P, P, None, 2, 8, 32, 4, 128, 256, 16, 8192, 0.1, _lib.DT_BF16, P, P, need - 1, None) == 5
     assert lib.odsd_paged_attention_workspace_bytes(2, 8, 32, 4, 96, 256, 16) == 0
+    # more query rows per (sequence, KV head) than the launch grid holds: refused, not truncated
+    assert att(P, P, P, P, P, None, 1, 600000, 32, 4, 128, 256, 16, 8192, 0.1, _lib.DT_BF16, P, P, 1 << 30, None) == 3
+    assert lib.odsd_paged_attention_workspace_bytes(1, 600000, 32, 4, 128, 256, 16) == 0
     # many sequences: one workgroup per (sequence, KV head) walks all its keys, no partial results
     assert lib.odsd_paged_attention_workspace_bytes(512, 1, 32, 4, 128, 256, 16) == 256
     # variable-length (prefill) attention: q, k, v, cu_q, cu_k, n_seqs, max_q, max_k, H, KVH, HD, scale, dtype,
