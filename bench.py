@@ -85,20 +85,31 @@ def _stage_stats(per_step):
     return [sum(s[k] for s in per_step) / n for k in range(len(per_step[0]))]
 
 
-def _traffic(wl_name):
+def _traffic(wl_name, kernel=None):
     """HBM bytes per launch of the dominant kernel as measured offline with rocprofv3 --pmc
     (FETCH_SIZE, WRITE_SIZE) and recorded, with the commit it was measured on, in
     profiles/hbm_traffic.json; None when there is no record for the workload."""
     try:
         rec = json.load(open(TRAFFIC_FILE))[wl_name]
+        if kernel and not rec.get("kernel", "").startswith(kernel):
+            return None, None          # measured on another kernel than the one in use
         return rec["bytes_per_launch"], rec.get("commit")
     except (OSError, KeyError, ValueError):
         return None, None
 
 
-def _roofline(wl, kernel_ms, algorithmic_bytes):
+def _dominant(wl, k, active_experts, launches=1):
+    """The dominant kernel of a workload, its time per launch and the algorithmic bytes of one launch:
+    the one-launch expert kernel (gate_up + down weights of the active experts) where the library
+    uses it, the gate_up stream (two thirds of an expert's bytes) otherwise."""
+    if k.get("experts", 0.0) > 0.0:
+        return "w4_expert_fused_kernel", k["experts"] / launches, active_experts * wl.expert_w4_bytes / launches
+    return None, k["gate_up"] / launches, active_experts * (wl.expert_w4_bytes * 2 // 3) / launches
+
+
+def _roofline(wl, kernel_ms, algorithmic_bytes, kernel=None):
     gu_flops = 4 * wl.pairs * wl.H * wl.I
-    traffic, commit = _traffic(wl.name)
+    traffic, commit = _traffic(wl.name, kernel)
     if wl.regime == "prefill":
         ach = gu_flops / (kernel_ms * 1e-3) / 1e12
         roof = {"bound": "mfma", "kernel": "w4_gemm_prefill_kernel<gate_up>", "achieved": round(ach, 2),
@@ -106,7 +117,7 @@ def _roofline(wl, kernel_ms, algorithmic_bytes):
                 "traffic": traffic, "algorithmic_flops": gu_flops}
     else:
         ach = algorithmic_bytes / (kernel_ms * 1e-3) / 1e9
-        roof = {"bound": "hbm", "kernel": "w4_gemm_kernel<gate_up>", "achieved": round(ach, 1),
+        roof = {"bound": "hbm", "kernel": kernel or "w4_gemm_kernel<gate_up>", "achieved": round(ach, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4),
                 "traffic": traffic, "algorithmic_bytes": int(algorithmic_bytes)}
     if commit:
@@ -178,7 +189,7 @@ def bench_layer(wl, dev, steps, warmup, with_cpu):
     engine_ms = (time.perf_counter() - t0) * 1e3 / steps
 
     k = dict(zip(_lib.KERNEL_NAMES, stage_ms))
-    gu_bytes = active * (wl.expert_w4_bytes * 2 // 3)
+    dom_kernel, dom_ms, dom_bytes = _dominant(wl, k, active)
     res = {
         "workload": wl.name, "T": wl.T, "H": wl.H, "E": wl.E, "K": wl.K, "I": wl.I,
         "tokens_per_s": round(wl.T / (ms * 1e-3), 1), "ms_per_step": round(ms, 5),
@@ -188,7 +199,7 @@ def bench_layer(wl, dev, steps, warmup, with_cpu):
         "layer_mfma_frac": round(wl.algorithmic_flops() / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
         "kernel_ms": {n: round(v, 5) for n, v in k.items()},
         "kernel_ms_sum": round(sum(stage_ms), 5),
-        "roofline": _roofline(wl, k["gate_up"], gu_bytes),
+        "roofline": _roofline(wl, dom_ms, dom_bytes, dom_kernel),
     }
     del runner, placements, plan, banks, tables
     if with_cpu:
@@ -255,7 +266,7 @@ def bench_stack(wl, dev, steps, warmup, with_cpu, cpu_layers=4):
     k = dict(zip(_lib.KERNEL_NAMES, stage_ms))
     # active experts per layer: re-run the layers' routing through the whole-block outputs
     active = _stack_active_experts(stack, x, wl)
-    gu_bytes_total = sum(active) * (wl.expert_w4_bytes * 2 // 3)
+    dom_kernel, dom_ms, dom_bytes = _dominant(wl, k, sum(active), wl.layers)
     alg_bytes = sum(wl.algorithmic_bytes(a, out_bytes=2) for a in active)
     res = {
         "workload": wl.name, "T": wl.T, "H": wl.H, "E": wl.E, "K": wl.K, "I": wl.I, "layers": wl.layers,
@@ -269,7 +280,7 @@ def bench_stack(wl, dev, steps, warmup, with_cpu, cpu_layers=4):
         "kernel_ms_sum": round(sum(stage_ms), 5),
         "kernel_ms_note": f"sums over the {wl.layers} layers of one step",
         # the dominant kernel runs once per layer: average launch = sum over layers / layers
-        "roofline": _roofline(wl, k["gate_up"] / wl.layers, gu_bytes_total / wl.layers),
+        "roofline": _roofline(wl, dom_ms, dom_bytes, dom_kernel),
     }
     del stack, events
     if with_cpu:

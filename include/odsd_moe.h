@@ -47,7 +47,7 @@ extern "C" {
 #endif
 
 /* 110: events / static forms of the whole block, KV store, paged and packed attention added (100: the MoE block) */
-#define ODSD_VERSION 110
+#define ODSD_VERSION 111
 
 typedef enum odsd_status {
     ODSD_OK = 0,
@@ -275,7 +275,9 @@ enum {
     ODSD_KERNEL_GATE_UP = 4,
     ODSD_KERNEL_DOWN = 5,
     ODSD_KERNEL_COMBINE = 6,
-    ODSD_N_KERNELS = 7
+    ODSD_KERNEL_EXPERTS = 7,        /* gate_up + SiLU*mul + down as one launch (shapes with many
+                                       small experts; slots 4 and 5 are then left out)          */
+    ODSD_N_KERNELS = 8
 };
 int odsd_moe_forward_events(const odsd_moe_shape *s, const void *x, const void *norm_weight,
                             float eps, const void *gate_w, const uint64_t *table,

@@ -68,8 +68,8 @@ SIGNATURES = {
                                           _P, _P, _P, _P, _P]),
 }
 
-N_KERNELS = 7                          # ODSD_N_KERNELS
-KERNEL_NAMES = ("norm", "router_logits", "router_topk", "dispatch", "gate_up", "down", "combine")
+N_KERNELS = 8                          # ODSD_N_KERNELS
+KERNEL_NAMES = ("norm", "router_logits", "router_topk", "dispatch", "gate_up", "down", "combine", "experts")
 STATIC_SCRATCH_BYTES = 64 << 20        # ODSD_STATIC_SCRATCH_BYTES
 
 _lib: Optional[C.CDLL] = None

@@ -369,7 +369,8 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
 // and weight first, then KB independent row loads -- and added in k order; with the generic loop
 // every row load waits for the one before it (its address hangs on a branch), which is what the
 // kernel's time consists of at K = 8.
-template <typename XT, bool YH, bool STATS, int KB>
+// YH: 0 = y holds fp32 partial sums; 1 = fp16 values in KS slices; 2 = exactly two fp16 slices
+template <typename XT, int YH, bool STATS, int KB>
 __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ y, const int32_t *__restrict__ idx,
                                                       const float *__restrict__ w,
                                                       const int32_t *__restrict__ perm,
@@ -405,14 +406,34 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
                     slot[u] = ok[u] ? sl : 0;      // a row that exists; its values are discarded below
                 }
                 float4_t v[KB > 0 ? KB : 1];
+                if (YH == 2) {
+                    // two fp16 slices: all 2 KB row loads are issued before the first is used
+                    half4_t h0[KB > 0 ? KB : 1], h1[KB > 0 ? KB : 1];
+#pragma unroll
+                    for (int u = 0; u < KB; ++u) {
+                        h0[u] = *(const half4_t *)((const half_t *)y + (size_t)slot[u] * H + c);
+                        h1[u] = *(const half4_t *)((const half_t *)y + ((size_t)P + slot[u]) * H + c);
+                    }
+#pragma unroll
+                    for (int u = 0; u < KB; ++u) {
+                        v[u] = float4_t{(float)h0[u].x, (float)h0[u].y, (float)h0[u].z, (float)h0[u].w};
+                        v[u] += float4_t{(float)h1[u].x, (float)h1[u].y, (float)h1[u].z, (float)h1[u].w};
+                    }
+                } else {
 #pragma unroll
                 for (int u = 0; u < KB; ++u) {
                     if (YH) {
                         const half4_t hv = *(const half4_t *)((const half_t *)y + (size_t)slot[u] * H + c);
                         v[u] = float4_t{(float)hv.x, (float)hv.y, (float)hv.z, (float)hv.w};
+                        // fp16 partial sums of further slices of the reduction, added in slice order
+                        for (int s = 1; s < KS; ++s) {
+                            const half4_t hs = *(const half4_t *)((const half_t *)y + ((size_t)s * P + slot[u]) * H + c);
+                            v[u] += float4_t{(float)hs.x, (float)hs.y, (float)hs.z, (float)hs.w};
+                        }
                     } else {
                         v[u] = *(const float4_t *)(y + (size_t)slot[u] * H + c);
                     }
+                }
                 }
 #pragma unroll
                 for (int u = 0; u < KB; ++u) {
@@ -432,9 +453,13 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
             if (slot < 0 || e < 0 || e >= E || table[(size_t)e * ODSD_TABLE_COLS] == 0) continue;
             float4_t v;
             if (YH) {
-                // prefill shapes: one fp16 value per output (KS == 1)
+                // fp16 values: complete sums (KS == 1) or the partial sums of KS slices
                 const half4_t hv = *(const half4_t *)((const half_t *)y + (size_t)slot * H + c);
                 v = float4_t{(float)hv.x, (float)hv.y, (float)hv.z, (float)hv.w};
+                for (int s = 1; s < KS; ++s) {
+                    const half4_t hs = *(const half4_t *)((const half_t *)y + ((size_t)s * P + slot) * H + c);
+                    v += float4_t{(float)hs.x, (float)hs.y, (float)hs.z, (float)hs.w};
+                }
             } else {
                 v = *(const float4_t *)(y + (size_t)slot * H + c);
                 for (int s = 1; s < KS; ++s) v += *(const float4_t *)(y + ((size_t)s * P + slot) * H + c);
@@ -483,8 +508,14 @@ struct ExpertsPlan {
     int PS_gu, PS_dn;  // prefill tile kernel: workgroups sharing the row passes of one tile
     int tile;        // MB == 8: the 256 x 256 tile kernel instead of the streaming kernel
     int y_f16;       // down-projection outputs kept as fp16 (unsplit reduction) instead of fp32 partials
+    int fused;       // whole-block calls run gate_up and down as one launch (experts_fused.hip)
+    int S;           // fused: workgroups per expert = fp16 partial-sum slices of the down projection
     size_t h_bytes, y_bytes;
 };
+
+// one-launch expert kernel (experts_fused.hip)
+void odsd_launch_experts_fused(FusedParams &fp, int E, hipStream_t st);
+int odsd_fused_supported(int H, int I, int S);
 
 // Choices are functions of the shape only (the per-expert counts live on the device).
 static ExpertsPlan experts_plan(const odsd_moe_shape *s) {
@@ -550,6 +581,21 @@ static ExpertsPlan experts_plan(const odsd_moe_shape *s) {
     p.y_f16 = p.KS == 1;
     p.h_bytes = odsd_round_up((size_t)(P > 0 ? P : 1) * s->I * sizeof(half_t), 256);
     p.y_bytes = odsd_round_up((size_t)p.KS * (size_t)(P > 0 ? P : 1) * s->H * sizeof(float), 256);
+    // The one-launch expert kernel serves calls where nearly every expert has rows and a pass holds
+    // them all (8 to 16 rows per expert on average, at most 32 per pass): one workgroup per
+    // (expert, slice of the intermediate dimension), E * S workgroups for 256 CUs.  The stage entry
+    // points keep the two-launch plan above; only the whole-block calls take this path.
+    p.fused = 0;
+    p.S = 1;
+    if (p.MB == 2 && s->T > 16 && mean_rows >= 8) {
+        int S = 256 / s->E;
+        if (S >= 1 && S <= 4 && s->E * S >= 192 && odsd_fused_supported(s->H, s->I, S)) {
+            p.fused = 1;
+            p.S = S;
+            const size_t need = odsd_round_up((size_t)S * (size_t)P * s->H * sizeof(half_t), 256);
+            if (need > p.y_bytes) p.y_bytes = need;
+        }
+    }
     return p;
 }
 
@@ -658,9 +704,11 @@ extern "C" int odsd_w4_down(const odsd_moe_shape *s, const void *h_f16, const ui
 }
 
 // combine: y partials + routing weights (+ residual) -> out (+ per-row sum of squares of out_act)
+// y_slices > 0: y holds that many fp16 partial-sum slices [slice][P][H] (the one-launch expert kernel);
+// 0: the layout of the two-launch plan
 static int launch_combine(const odsd_moe_shape *s, const void *y_, const int32_t *idx, const float *w,
                           const int32_t *perm, const uint64_t *table, const void *residual,
-                          float *out_f32, void *out_act, double *row_ss, hipStream_t st) {
+                          float *out_f32, void *out_act, double *row_ss, hipStream_t st, int y_slices = 0) {
     const int rc = experts_args_ok(s);
     if (rc != ODSD_OK) return rc;
     if (s->T == 0) return ODSD_OK;
@@ -669,12 +717,13 @@ static int launch_combine(const odsd_moe_shape *s, const void *y_, const int32_t
     if (!out_f32 && !out_act) return ODSD_ERR_NULL;
     if (row_ss && !out_act) return ODSD_ERR_NULL;
     if (!odsd_aligned16(y) || (out_f32 && !odsd_aligned16(out_f32))) return ODSD_ERR_ALIGN;
-    const ExpertsPlan pl = experts_plan(s);
+    ExpertsPlan pl = experts_plan(s);
+    if (y_slices > 0) { pl.KS = y_slices; pl.y_f16 = 1; }
     const int P = s->T * s->K;
     const int nchunk = (s->H / 4 + 255) / 256;
     if ((int64_t)nchunk * s->T > 0x7fffffffLL) return ODSD_ERR_UNSUPPORTED;
     const dim3 grid((unsigned)(nchunk * s->T));
-    const bool batched = pl.KS == 1 && s->K % 4 == 0;      // rows of 4 pairs fetched together (8: no faster)
+    const bool batched = (pl.KS == 1 || pl.y_f16) && s->K % 4 == 0;      // rows of 4 pairs fetched together (8: no faster)
 #define COMBINE_GO(XT, YH, ST)                                                                          \
     do {                                                                                                \
         if (batched)                                                                                    \
@@ -686,10 +735,11 @@ static int launch_combine(const odsd_moe_shape *s, const void *y_, const int32_t
                         table, (const XT *)residual, out_f32, (XT *)out_act, row_ss, s->T, s->H, s->K,  \
                         s->E, pl.KS, P, nchunk);                                                        \
     } while (0)
-#define COMBINE_Y(XT, ST)                          \
-    do {                                           \
-        if (pl.y_f16) COMBINE_GO(XT, true, ST);    \
-        else COMBINE_GO(XT, false, ST);            \
+#define COMBINE_Y(XT, ST)                                    \
+    do {                                                     \
+        if (pl.y_f16 && pl.KS == 2) COMBINE_GO(XT, 2, ST);   \
+        else if (pl.y_f16) COMBINE_GO(XT, 1, ST);            \
+        else COMBINE_GO(XT, 0, ST);                          \
     } while (0)
     if (s->act_dtype == ODSD_DT_BF16) {
         if (row_ss) COMBINE_Y(uint16_t, true);
@@ -723,6 +773,18 @@ int odsd_launch_experts(const odsd_moe_shape *s, const void *x16, const uint64_t
     if (ws_bytes < pl.h_bytes + pl.y_bytes) return ODSD_ERR_WORKSPACE;
     void *h16 = ws;
     float *y = (float *)((char *)ws + pl.h_bytes);
+    if (pl.fused) {
+        if (!x16 || !table || !counts || !offsets || !slot_token) return ODSD_ERR_NULL;
+        if (!odsd_aligned16(x16)) return ODSD_ERR_ALIGN;
+        FusedParams fp{};
+        fp.table = table; fp.x16 = (const half_t *)x16; fp.rowmap = slot_token;
+        fp.counts = counts; fp.offsets = offsets; fp.y = (half_t *)y;
+        fp.H = s->H; fp.I = s->I; fp.S = pl.S; fp.P = s->T * s->K;
+        fp.G_up = s->H / ODSD_GROUP; fp.G_dn = s->I / ODSD_GROUP;
+        odsd_launch_experts_fused(fp, s->E, st);
+        ODSD_CHECK_LAUNCH();
+        return launch_combine(s, y, idx, w, perm, table, residual, out_f32, out_act, row_ss, st, pl.S);
+    }
     rc = odsd_w4_gate_up_silu(s, x16, table, counts, offsets, slot_token, h16, st);
     if (rc != ODSD_OK) return rc;
     rc = odsd_w4_down(s, h16, table, counts, offsets, y, st);

@@ -1,0 +1,270 @@
+// One launch per MoE block for the experts of verify-shaped calls on models with many small
+// experts (Qwen3-30B-A3B: hidden 2048, 128 experts of intermediate 768, 8-32 rows per expert).
+//
+// The two-launch form (w4_gemm_kernel, MODE 0 then MODE 1) moves as many token-row bytes
+// L2 -> LDS as it streams weight bytes from HBM -- every workgroup copies its expert's rows for
+// every 128-column group, with a barrier per group -- and pays a launch ramp twice.  Here one
+// workgroup of 8 wavefronts owns (expert, slice s of S of the intermediate features) for the
+// whole block:
+//   * the expert's token rows (at most 16*MB rows x H fp16 = 128 KB) are copied into LDS ONCE,
+//     by asynchronous global -> LDS loads, in the B-fragment order of v_mfma_f32_16x16x32_f16
+//     ([group][token block][16 rows x 256 B], 16-byte segments XOR-swizzled by the row);
+//   * gate_up: each wavefront owns whole (gate block, up block) pairs of the slice and walks them
+//     pair after pair, group after group: one step = the two 1 KiB tiles of one group, fetched by
+//     buffer loads through a register ring 4 steps deep (two ascending 16 KiB runs per pair),
+//     expanded int4 -> fp16 in registers and multiplied with the group's fragments read from LDS;
+//     no barrier in the stream;
+//   * h = SiLU(gate) * up of a pair (16*MB rows x 16 features, fp16) goes to LDS in the same
+//     fragment order when the pair's last group is done; one barrier after the last pair;
+//   * down: the same stream over pairs of output row blocks, the slice's GS groups of each (the
+//     ring runs on from gate_up into down without draining), against h from LDS; fp16 partial sums
+//     y[s][slot][H] are stored per pair; the combine adds the S slices in order.
+// Workgroups hold 152 KB of LDS, so exactly one is resident per CU: E*S is chosen near the CU
+// count and every workgroup streams the same number of bytes.
+//
+// Replaces the same reference code as the streaming kernels: the three F.linear calls of
+// expert_forward_with_weights (demo/src/layers/mlp.py:227-230) inside the per-expert loop of
+// demo/src/model/qwen3_runner.py:303-380.
+#include "w4_gemm.h"
+
+#include <type_traits>
+
+// MB    16-row token blocks held per pass (an expert with more rows takes further passes)
+// GS    128-column groups of the intermediate dimension per slice (slice = 128*GS features)
+// WAVES wavefronts per workgroup
+// G_UP  H / 128, G_DN  I / 128: groups of the two reductions (compile time: every tile offset of
+//       a wavefront's stream is a constant)
+template <int MB, int GS, int WAVES, int G_UP, int G_DN>
+__global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(const FusedParams p) {
+    static_assert(WAVES % 4 == 0 && (8 * GS) % WAVES == 0, "whole gate/up block pairs per wavefront");
+    static_assert(G_UP * MB <= ODSD_FUSED_X_BLOCKS, "token rows of a pass must fit the LDS area");
+    static_assert(MB == 1 || MB == 2, "one or two token blocks");
+    constexpr int PPW = 8 * GS / WAVES;          // gate/up block pairs per wavefront
+    constexpr int NT = PPW * G_UP;               // gate_up steps of a wavefront: pair after pair, group after group
+    constexpr int DPAIRS = G_UP * 4;             // pairs of down row blocks: H / 32
+    constexpr int DP_MIN = DPAIRS / WAVES, DP_EXTRA = DPAIRS % WAVES;   // the first DP_EXTRA wavefronts take one more
+    constexpr int NTD = (DP_MIN + (DP_EXTRA ? 1 : 0)) * GS;             // most down steps any wavefront runs
+    constexpr int DEPTH = 4;                     // ring: steps (two tiles each) in flight
+    constexpr int XBLK = 4096;                   // bytes of one (group, token block): 16 rows x 256 B
+    static_assert(NT >= DEPTH && DP_MIN * GS >= DEPTH, "ring deeper than a stream");
+    __shared__ __attribute__((aligned(16))) char xs_raw[ODSD_FUSED_X_BLOCKS * XBLK];
+    __shared__ __attribute__((aligned(16))) char hs_raw[GS * MB * XBLK];
+
+    const int b = blockIdx.x;
+    const int e = b / p.S, s = b - e * p.S;
+    // everything the prologue depends on is requested at once (one round trip, not three)
+    const uint64_t *trow = p.table + (size_t)e * ODSD_TABLE_COLS;
+    const int M_e = p.counts[e];
+    const int base = p.offsets[e];
+    const uint64_t t_gu_q = trow[0], t_gu_sz = trow[1], t_dn_q = trow[2], t_dn_sz = trow[3];
+    if (M_e == 0 || t_gu_q == 0) return;
+    const global_char *src_c = (const global_char *)p.x16;
+    // the expert's packed matrices and their (scale, zero) pairs as buffer resources (reads past
+    // the end return zero)
+    const __amdgpu_buffer_rsrc_t rsrc_qu = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(uintptr_t)t_gu_q, 0, (2 * p.I / 16) * G_UP * 1024, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_szu = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(uintptr_t)t_gu_sz, 0, (2 * p.I / 16) * G_UP * 64, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_qd = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(uintptr_t)t_dn_q, 0, (p.H / 16) * G_DN * 1024, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_szd = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(uintptr_t)t_dn_sz, 0, (p.H / 16) * G_DN * 64, 0x00020000);
+
+    const DequantConsts dc = dequant_consts();
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, kq = lane >> 4;
+
+    // gate_up duty: block pairs of the slice (the slice owns the fused matrix's blocks
+    // s*16*GS .. (s+1)*16*GS - 1).  A pair is 2 * G_UP KiB of contiguous tiles -- [gate block][group],
+    // then [up block][group] -- and the wavefront walks it group by group, so it reads two ascending
+    // runs of G_UP KiB; tile (pair i, block j, group g) sits at the compile-time offset
+    // ((2 i + j) * G_UP + g) KiB from the wavefront's first tile.
+    const int ublk0 = s * (16 * GS) + wave * (2 * PPW);
+    const uint32_t uq_off = ((uint32_t)ublk0 * G_UP * 64 + lane) * 16u;
+    const uint32_t usz_off = ((uint32_t)ublk0 * G_UP * 16 + r) * 4u;
+    // down duty: pairs of output row blocks; of each block's G_DN tiles the slice reads the GS
+    // contiguous ones from s*GS on
+    const int npairs_w = DP_MIN + (wave < DP_EXTRA ? 1 : 0);
+    const int ntd_w = npairs_w * GS;
+    const int dblk0 = 2 * (wave * DP_MIN + min(wave, DP_EXTRA));
+    const uint32_t dq_off = (((uint32_t)dblk0 * G_DN + s * GS) * 64 + lane) * 16u;
+    const uint32_t dsz_off = (((uint32_t)dblk0 * G_DN + s * GS) * 16 + r) * 4u;
+
+    // LDS byte offset of this lane's B fragment of 32-column step j inside a (group, token block):
+    // row r, logical segment 4j + kq, stored at segment ^ r
+    uint32_t lds_frag[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) lds_frag[j] = (uint32_t)((r * 16 + ((4 * j + kq) ^ r)) * 16);
+
+    // token-row copies: one copy instruction moves 4 rows x 256 B (lane -> row lane / 16, stored
+    // segment lane % 16).  A wavefront always copies the same quarter of the same token block, for
+    // one group per instruction, so it needs one source row per lane.
+    // (the first 8 wavefronts copy; the others have none)
+    const int quarter = wave & 3;
+    const int dm = MB == 2 ? ((wave >> 2) & 1) : 0;           // token block this wavefront copies
+    const int row_in_blk = 4 * quarter + kq;
+    constexpr int N_PIECES = G_UP * MB / 2;                   // copies per wavefront
+
+    for (int m0 = 0; m0 < M_e; m0 += 16 * MB) {
+        const int mcnt = min(M_e - m0, 16 * MB);
+        const int nmb = scalar_int((mcnt + 15) >> 4);
+        __syncthreads();                                      // the previous pass is done with both LDS areas
+
+        // One ring for both phases: slot = step % DEPTH holds the two tiles of a step.
+        uint4_t wq[DEPTH][2];
+        uint32_t wsz[DEPTH][2];
+        auto load_u = [&](const int slot, const int t) {      // gate_up step t
+            const int tile = 2 * (t / G_UP) * G_UP + t % G_UP;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                wq[slot][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_qu, (int)uq_off, (tile + i * G_UP) * 1024, 2 /* nt */);
+                wsz[slot][i] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_szu, (int)usz_off, (tile + i * G_UP) * 64, 0);
+            }
+        };
+        auto load_d = [&](const int slot, const int u) {      // down step u
+            const int tile = 2 * (u / GS) * G_DN + u % GS;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                wq[slot][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_qd, (int)dq_off, (tile + i * G_DN) * 1024, 2 /* nt */);
+                wsz[slot][i] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_szd, (int)dsz_off, (tile + i * G_DN) * 64, 0);
+            }
+        };
+        // the ring's first loads depend on the table row only: they travel while the row map is
+        // read and the token rows are copied
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) load_u(d, d);
+        // rows past the expert's last one are clamped to the first row of the pass: the MFMA
+        // columns they feed are never stored
+        {
+            const int row = dm * 16 + row_in_blk;
+            const int slot = base + m0 + (row < mcnt ? row : 0);
+            const int srow = p.rowmap[slot];
+            const uint32_t st_off = ((uint32_t)srow * (uint32_t)p.H + (uint32_t)((r ^ row_in_blk) * 8)) * 2u;
+            if (dm < nmb && wave < 8) {
+                for (int i = 0; i < N_PIECES; ++i) {
+                    const int g = MB == 2 ? i : 2 * i + ((wave >> 2) & 1);
+                    lds_void *dst = (lds_void *)(xs_raw + (g * MB + dm) * XBLK + quarter * 1024);
+                    dma16_to_lds(src_c + (size_t)g * (ODSD_GROUP * 2u), st_off, dst);
+                }
+            }
+        }
+        ODSD_WAIT_VMCNT(0);                                   // the copies are the youngest requests
+        __builtin_amdgcn_s_barrier();
+
+        // One step = one group of one block pair: B fragments of the group from LDS, the slot's two
+        // tiles expanded to fp16, the slot refilled with the step DEPTH ahead, 2 x MB x 4 MFMAs.
+        // Both streams of a wavefront are unrolled: ring slots, tile offsets and LDS addresses are
+        // constants, and the wait the compiler derives for a slot leaves the younger slots in flight.
+        float4_t acc[2][MB];
+        auto step = [&](const int slot, const char *frag_base, auto refill) {
+            half8_t bx[MB][4];
+#pragma unroll
+            for (int m = 0; m < MB; ++m) {
+                if (m == 0 || m < nmb) {                      // (a pass has at least one row)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) bx[m][j] = *(const half8_t *)(frag_base + m * XBLK + lds_frag[j]);
+                }
+            }
+            half8_t a[2][4];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) dequant_tile(dc, wq[slot][i], wsz[slot][i], a[i]);
+            __builtin_amdgcn_sched_barrier(0);
+            refill();                                         // the slot is free again
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int m = 0; m < MB; ++m) {
+                if (m == 0 || m < nmb) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+#pragma unroll
+                        for (int i = 0; i < 2; ++i) acc[i][m] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i][j], bx[m][j], acc[i][m], 0, 0, 0);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        auto zero_acc = [&]() {
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int m = 0; m < MB; ++m) acc[i][m] = float4_t{0.f, 0.f, 0.f, 0.f};
+        };
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            const int pi = t / G_UP, g = t % G_UP;
+            if (g == 0) zero_acc();
+            step(t % DEPTH, xs_raw + (g * MB) * XBLK, [&]() {
+                // past the end of gate_up the ring goes on with the first steps of the down stream
+                if (t + DEPTH < NT) load_u(t % DEPTH, t + DEPTH);
+                else if (t + DEPTH - NT < ntd_w) load_d(t % DEPTH, t + DEPTH - NT);
+            });
+            if (g == G_UP - 1 || t == NT - 1) {
+                // h = SiLU(gate) * up of this pair's 16 features -> LDS, in fragment order: the lane
+                // holds features 4*kq .. 4*kq+3 of token column r
+                const int fbl = wave * PPW + pi;             // 16-feature block inside the slice
+                const int gl = fbl >> 3, seg = (fbl & 7) * 2 + (kq >> 1);
+#pragma unroll
+                for (int m = 0; m < MB; ++m) {
+                    if (m == 0 || m < nmb) {
+                        const float4_t gt = acc[0][m], up = acc[1][m];
+                        half4_t h;
+                        h.x = f32_to_f16_sat(silu_f32(gt.x) * up.x);
+                        h.y = f32_to_f16_sat(silu_f32(gt.y) * up.y);
+                        h.z = f32_to_f16_sat(silu_f32(gt.z) * up.z);
+                        h.w = f32_to_f16_sat(silu_f32(gt.w) * up.w);
+                        char *dst = hs_raw + (gl * MB + m) * XBLK + r * 256 + ((seg ^ r) * 16) + (kq & 1) * 8;
+                        *(half4_t *)dst = h;
+                    }
+                }
+            }
+        }
+        __syncthreads();                                      // h is complete
+
+        // down: step u = group u % GS of output block pair u / GS, against h from LDS; the slice's
+        // partial sums are stored as fp16 when a pair's last group is done
+#pragma unroll
+        for (int u = 0; u < NTD; ++u) {
+            if (u >= DP_MIN * GS && u >= ntd_w) break;
+            const int pi = u / GS, gl = u % GS;
+            if (gl == 0) zero_acc();
+            step((NT + u) % DEPTH, hs_raw + (gl * MB) * XBLK, [&]() {
+                if (u + DEPTH < NTD && u + DEPTH < ntd_w) load_d((NT + u) % DEPTH, u + DEPTH);
+            });
+            if (gl == GS - 1) {
+                // lane holds outputs 4*kq .. 4*kq+3 of each block, token column r
+#pragma unroll
+                for (int m = 0; m < MB; ++m) {
+                    const int row = m * 16 + r;
+                    if (m < nmb && row < mcnt) {
+                        const size_t slot = (size_t)(base + m0 + row);
+                        half_t *yrow = p.y + ((size_t)s * p.P + slot) * p.H;
+#pragma unroll
+                        for (int i = 0; i < 2; ++i) {
+                            const int n = (dblk0 + 2 * pi + i) * 16 + kq * 4;
+                            const float4_t v = acc[i][m];
+                            *(half4_t *)(yrow + n) =
+                                half4_t{f32_to_f16_sat(v.x), f32_to_f16_sat(v.y), f32_to_f16_sat(v.z), f32_to_f16_sat(v.w)};
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+// Shapes the fused kernel is built for; the caller has checked them with odsd_fused_supported().
+void odsd_launch_experts_fused(FusedParams &fp, int E, hipStream_t st) {
+    // (MB = 2: up to 32 rows per pass; experts with at most 16 rows skip the second token block)
+    ODSD_LAUNCH(ODSD_KERNEL_EXPERTS, (w4_expert_fused_kernel<2, 3, 8, 16, 6>), E * fp.S, 512, st, fp);
+}
+
+// H = 2048 (4 sub-passes of 8 wavefronts x 4 blocks), slices of 384 features, token rows of one
+// pass within the 128 KB row area
+int odsd_fused_supported(int H, int I, int S) {
+    if (S < 1 || I % (ODSD_GROUP * S)) return 0;
+    if (I / (ODSD_GROUP * S) != 3 || I / ODSD_GROUP != 6) return 0;
+    if (H != 2048) return 0;
+    if ((H / ODSD_GROUP) * 2 > ODSD_FUSED_X_BLOCKS) return 0;
+    return 1;
+}

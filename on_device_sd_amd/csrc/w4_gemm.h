@@ -31,6 +31,21 @@ struct GemmParams {
     int wg_per_xcd;          // ceil(n_wg / 8)
 };
 
+// Launch parameters of the one-launch expert kernel (experts_fused.hip)
+#define ODSD_FUSED_X_BLOCKS 32   // (group, token block) areas of 4 KiB in its token-row LDS area
+struct FusedParams {
+    const uint64_t *table;   // [E][4]
+    const half_t *x16;       // activations, fp16 [T][H]
+    const int32_t *rowmap;   // slot -> token
+    const int32_t *counts;
+    const int32_t *offsets;
+    half_t *y;               // [S][P][H] fp16 partial sums of the down projection
+    int H, I;
+    int S;                   // slices of the intermediate dimension (workgroups per expert)
+    int P;
+    int G_up, G_dn;          // H / 128, I / 128
+};
+
 __device__ __forceinline__ half2_t as_half2(uint32_t u) { return __builtin_bit_cast(half2_t, u); }
 
 // Constants of the code -> fp16 bit trick.  (x & mask) | magic is one VOP3 instruction

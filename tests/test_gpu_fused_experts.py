@@ -1,0 +1,108 @@
+"""The one-launch expert kernel (gate_up -> SiLU*mul -> down in one workgroup per expert slice).
+
+It serves whole-block calls at the Qwen3-30B-A3B expert shape (hidden 2048, 128 experts, top 8,
+intermediate 768) with 8 to 16 rows per expert on average; the stage entry points keep the
+two-launch plan.  The same hand-built routing goes through both, and through the CPU oracle:
+experts without rows, with exactly 16 / 17 / 32 / 33 rows (one and two token blocks, one and two
+passes) and one with 70 rows (three passes).  Replaces expert_forward_with_weights
+(demo/src/layers/mlp.py:227-230) inside the per-expert loop of qwen3_runner.py:303-380."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_oracle as orc
+from tests.helpers import canon_to_oracle, check_output, check_output_relative
+
+pytestmark = pytest.mark.gpu
+
+H, E, K, I = 2048, 128, 8, 768
+
+
+@pytest.fixture(scope="module")
+def layer(dev):
+    import on_device_sd_amd as odsd
+    g = torch.Generator().manual_seed(11)
+    bank = odsd.W4ExpertBank(E, H, I, dev)
+    experts = {}
+    for e in range(E):
+        canon = bank.load_expert(e, torch.randn(I, H, generator=g) * 0.02, torch.randn(I, H, generator=g) * 0.02,
+                                 torch.randn(H, I, generator=g) * 0.02, keep_canonical=True)
+        experts[e] = canon_to_oracle(canon)
+    return bank, experts
+
+
+def _routing(T, forced, seed):
+    """[T, K] expert ids: expert e of `forced` gets exactly forced[e] rows (0 = none), the other
+    pairs are spread over the remaining experts; ids inside a token are distinct."""
+    rng = np.random.default_rng(seed)
+    idx = -np.ones((T, K), dtype=np.int64)
+    fill = np.zeros(T, dtype=np.int64)
+    for e, n in forced.items():
+        cand = np.flatnonzero(fill < K)
+        toks = rng.choice(cand, size=n, replace=False)
+        for t in toks:
+            idx[t, fill[t]] = e
+            fill[t] += 1
+    free = np.array([e for e in range(E) if e not in forced])
+    for t in range(T):
+        need = K - fill[t]
+        if need:
+            idx[t, fill[t]:] = rng.choice(free, size=need, replace=False)
+    for t in range(T):
+        rng.shuffle(idx[t])
+    assert (idx >= 0).all()
+    return idx
+
+
+CASES = [
+    # T, {expert: rows}
+    (256, {}),                                                   # the benchmark's shape, uniform routing
+    (128, {}),                                                   # 8 rows per expert on average
+    (200, {0: 0, 1: 16, 2: 17, 3: 32, 4: 33, 5: 70, 6: 1, 127: 0}),
+]
+
+
+@pytest.mark.parametrize("T,forced", CASES)
+def test_fused_experts_vs_stages_and_oracle(dev, layer, T, forced):
+    print("fused experts", T, forced, flush=True)
+    from on_device_sd_amd import _lib, ops
+    import ctypes as C
+    bank, experts = layer
+    g = torch.Generator().manual_seed(T)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    idx_np = _routing(T, forced, seed=T)
+    w_np = np.random.default_rng(T + 1).random((T, K), dtype=np.float32)
+    w_np /= w_np.sum(axis=1, keepdims=True)
+    idx = torch.from_numpy(idx_np).to(torch.int32).to(dev)
+    w = torch.from_numpy(w_np).to(dev)
+    counts = np.bincount(idx_np.ravel(), minlength=E)
+    for e, n in forced.items():
+        assert counts[e] == n
+    x16 = ops.to_f16(x.to(dev))
+    disp = ops.dispatch(idx, E)
+    assert np.array_equal(disp.counts.cpu().numpy(), counts)
+
+    # whole-block call: the one-launch kernel (the plan says so for this shape)
+    out32, outa = ops.experts_w4(x16, bank.table(), idx, w, disp, I, torch.bfloat16, want_f32=True, want_act=True)
+    # stage by stage: the two-launch kernels on the same routing
+    st = ops.ExpertStages(T, H, E, K, I, torch.bfloat16, dev)
+    st.gate_up(x16, bank.table(), disp)
+    st.down(bank.table(), disp)
+    ref32 = torch.empty(T, H, dtype=torch.float32, device=dev)
+    st.combine(idx, w, disp, bank.table(), out_f32=ref32)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out32).all()
+    # the two differ by the fp16 rounding of the two partial sums of the down projection
+    d = (out32 - ref32).abs().max().item()
+    scale = ref32.abs().max().item()
+    print(f"  fused vs two-launch: max-abs {d:.3e} at max|out| {scale:.3e}", flush=True)
+    assert d <= 2e-3 * scale
+    # against the oracle, every token
+    ref = orc.moe_forward(x, idx_np, w_np, experts)
+    mx, mean = check_output(out32, ref)
+    check_output_relative(out32, ref)
+    print(f"  vs oracle: max-abs {mx:.3e} mean-abs {mean:.3e}", flush=True)
+    assert torch.equal(outa.cpu(), out32.cpu().to(torch.bfloat16))
+    # a second run gives the same bits
+    out32b, _ = ops.experts_w4(x16, bank.table(), idx, w, disp, I, torch.bfloat16, want_f32=True, want_act=False)
+    assert torch.equal(out32b, out32)
