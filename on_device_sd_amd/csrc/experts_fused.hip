@@ -11,15 +11,19 @@
 //     ([group][token block][16 rows x 256 B], 16-byte segments XOR-swizzled by the row);
 //   * gate_up: each wavefront owns whole (gate block, up block) pairs of the slice and walks them
 //     pair after pair, group after group: one step = the two 1 KiB tiles of one group, fetched by
-//     buffer loads through a register ring 4 steps deep (two ascending 16 KiB runs per pair),
-//     expanded int4 -> fp16 in registers and multiplied with the group's fragments read from LDS;
-//     no barrier in the stream;
+//     buffer loads through a register ring 4 steps deep (two ascending 16 KiB runs per pair) and
+//     multiplied with the group's fragments read from LDS; no barrier in the stream;
+//   * the codes go to the matrix cores as they are (offset + q as fp16, two logic instructions per
+//     4 weights); the offsets leave through the accumulator's start value, and scale and zero point
+//     are applied to each group's sum, acc += scale * (sum q x - zero * sum x), in fp32 -- the
+//     per-weight (q - zero) * scale in fp16 is what the two-launch kernels spend most of their
+//     vector instructions on, and with one workgroup per CU this kernel is bound by those;
 //   * h = SiLU(gate) * up of a pair (16*MB rows x 16 features, fp16) goes to LDS in the same
 //     fragment order when the pair's last group is done; one barrier after the last pair;
 //   * down: the same stream over pairs of output row blocks, the slice's GS groups of each (the
 //     ring runs on from gate_up into down without draining), against h from LDS; fp16 partial sums
 //     y[s][slot][H] are stored per pair; the combine adds the S slices in order.
-// Workgroups hold 152 KB of LDS, so exactly one is resident per CU: E*S is chosen near the CU
+// Workgroups hold 157 KB of LDS, so exactly one is resident per CU: E*S is chosen near the CU
 // count and every workgroup streams the same number of bytes.
 //
 // Replaces the same reference code as the streaming kernels: the three F.linear calls of
@@ -28,6 +32,44 @@
 #include "w4_gemm.h"
 
 #include <type_traits>
+
+// Codes as fp16 without the per-weight scale and zero point.  (x & mask) | magic turns a nibble pair
+// into fp16 values offset + q: the low nibbles of the two halves of a word with magic 0x6400
+// (1024 + q, one unit in the last place = 1), the high nibbles with 0x5400 (64 + q, one unit in the
+// last place = 1/16, so the nibble's 16 q is q).  Element order of the result is that of the MFMA A
+// operand: (k0,k1) and (k4,k5) carry 1024 + q, (k2,k3) and (k6,k7) carry 64 + q.  The offsets are
+// taken out again through the accumulator's start value (see group_sums), and scale and zero point
+// are applied to the group's sum instead of to every weight: 5 vector instructions per 8 weights
+// instead of 13.
+struct RawConsts {
+    uint32_t m_lo, m_hi, magic_lo, magic_hi;
+};
+__device__ __forceinline__ RawConsts raw_consts() {
+    RawConsts c{0x000F000Fu, 0x00F000F0u, 0x64006400u, 0x54005400u};
+    asm volatile("" : "+s"(c.m_lo), "+s"(c.m_hi), "+v"(c.magic_lo), "+v"(c.magic_hi));
+    return c;
+}
+__device__ __forceinline__ half8_t raw_word(const RawConsts &c, const uint32_t x) {
+    const uint32_t xs = x >> 8;
+    const uint4_t t = {(x & c.m_lo) | c.magic_lo, (x & c.m_hi) | c.magic_hi, (xs & c.m_lo) | c.magic_lo,
+                       (xs & c.m_hi) | c.magic_hi};
+    return __builtin_bit_cast(half8_t, t);
+}
+#define ODSD_RAW_OFFSET_LO 1024.0f
+#define ODSD_RAW_OFFSET_HI 64.0f
+
+typedef float float2_t __attribute__((ext_vector_type(2)));
+
+// Nothing moves across this point: the scheduling fence binds the machine scheduler, the empty
+// statement with a memory clobber binds the instruction selector's ordering of a long straight-line
+// block (without it the loads of many later steps are hoisted to the top of the unrolled stream and
+// their results spilled).
+#define ODSD_FENCE()                         \
+    do {                                     \
+        __builtin_amdgcn_sched_barrier(0);   \
+        asm volatile("" ::: "memory");       \
+        __builtin_amdgcn_sched_barrier(0);   \
+    } while (0)
 
 // MB    16-row token blocks held per pass (an expert with more rows takes further passes)
 // GS    128-column groups of the intermediate dimension per slice (slice = 128*GS features)
@@ -49,6 +91,9 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
     static_assert(NT >= DEPTH && DP_MIN * GS >= DEPTH, "ring deeper than a stream");
     __shared__ __attribute__((aligned(16))) char xs_raw[ODSD_FUSED_X_BLOCKS * XBLK];
     __shared__ __attribute__((aligned(16))) char hs_raw[GS * MB * XBLK];
+    // per (group, token block) and token row: (sum of offset_k * x_k, sum of x_k) over the group's 128
+    // columns -- the token rows' blocks first, the blocks of h after them
+    __shared__ float2_t cx[(G_UP + GS) * MB * 16];
 
     const int b = blockIdx.x;
     const int e = b / p.S, s = b - e * p.S;
@@ -70,7 +115,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
     const __amdgpu_buffer_rsrc_t rsrc_szd = __builtin_amdgcn_make_buffer_rsrc(
         (void *)(uintptr_t)t_dn_sz, 0, (p.H / 16) * G_DN * 64, 0x00020000);
 
-    const DequantConsts dc = dequant_consts();
+    const RawConsts rc = raw_consts();
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -83,14 +128,16 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
     // ((2 i + j) * G_UP + g) KiB from the wavefront's first tile.
     const int ublk0 = s * (16 * GS) + wave * (2 * PPW);
     const uint32_t uq_off = ((uint32_t)ublk0 * G_UP * 64 + lane) * 16u;
-    const uint32_t usz_off = ((uint32_t)ublk0 * G_UP * 16 + r) * 4u;
+    // (scale, zero) pairs are fetched in accumulator order: the lane's 4 output rows 4*kq .. 4*kq+3 are
+    // 16 contiguous bytes of a tile's 64
+    const uint32_t usz_off = ((uint32_t)ublk0 * G_UP * 16 + 4 * kq) * 4u;
     // down duty: pairs of output row blocks; of each block's G_DN tiles the slice reads the GS
     // contiguous ones from s*GS on
     const int npairs_w = DP_MIN + (wave < DP_EXTRA ? 1 : 0);
     const int ntd_w = npairs_w * GS;
     const int dblk0 = 2 * (wave * DP_MIN + min(wave, DP_EXTRA));
     const uint32_t dq_off = (((uint32_t)dblk0 * G_DN + s * GS) * 64 + lane) * 16u;
-    const uint32_t dsz_off = (((uint32_t)dblk0 * G_DN + s * GS) * 16 + r) * 4u;
+    const uint32_t dsz_off = (((uint32_t)dblk0 * G_DN + s * GS) * 16 + 4 * kq) * 4u;
 
     // LDS byte offset of this lane's B fragment of 32-column step j inside a (group, token block):
     // row r, logical segment 4j + kq, stored at segment ^ r
@@ -109,18 +156,22 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
 
     for (int m0 = 0; m0 < M_e; m0 += 16 * MB) {
         const int mcnt = min(M_e - m0, 16 * MB);
-        const int nmb = scalar_int((mcnt + 15) >> 4);
         __syncthreads();                                      // the previous pass is done with both LDS areas
+        // The pass is compiled once per number of token blocks that hold rows: with a run-time count
+        // the values that exist on one path only (fragments, group sums, the second block's partial
+        // sums) stay live across the whole unrolled stream.
+        auto run_pass = [&](auto nmb_c) {
+        constexpr int nmb = decltype(nmb_c)::value;
 
         // One ring for both phases: slot = step % DEPTH holds the two tiles of a step.
         uint4_t wq[DEPTH][2];
-        uint32_t wsz[DEPTH][2];
+        uint4_t wsz[DEPTH][2];
         auto load_u = [&](const int slot, const int t) {      // gate_up step t
             const int tile = 2 * (t / G_UP) * G_UP + t % G_UP;
 #pragma unroll
             for (int i = 0; i < 2; ++i) {
                 wq[slot][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_qu, (int)uq_off, (tile + i * G_UP) * 1024, 2 /* nt */);
-                wsz[slot][i] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_szu, (int)usz_off, (tile + i * G_UP) * 64, 0);
+                wsz[slot][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_szu, (int)usz_off, (tile + i * G_UP) * 64, 0);
             }
         };
         auto load_d = [&](const int slot, const int u) {      // down step u
@@ -128,7 +179,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
 #pragma unroll
             for (int i = 0; i < 2; ++i) {
                 wq[slot][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_qd, (int)dq_off, (tile + i * G_DN) * 1024, 2 /* nt */);
-                wsz[slot][i] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_szd, (int)dsz_off, (tile + i * G_DN) * 64, 0);
+                wsz[slot][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_szd, (int)dsz_off, (tile + i * G_DN) * 64, 0);
             }
         };
         // the ring's first loads depend on the table row only: they travel while the row map is
@@ -153,36 +204,91 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
         ODSD_WAIT_VMCNT(0);                                   // the copies are the youngest requests
         __builtin_amdgcn_s_barrier();
 
+        // Sums of one (group, token block): the lane reads its four B fragments (token row r, columns
+        // 32 j + 8 kq ..), adds the values at the 1024-offset positions and at the 64-offset positions
+        // in fp32, the four kq parts are added across the lanes (same order in every lane), and the
+        // lanes of kq = 0 store (1024 * lo + 64 * hi, lo + hi) for their row.
+        auto group_sums = [&](const char *blk, float2_t *dst) {
+            float lo = 0.f, hi = 0.f;
+            const half2_t one = {(half_t)1.0f, (half_t)1.0f};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const half8_t f = *(const half8_t *)(blk + lds_frag[j]);
+                lo = __builtin_amdgcn_fdot2(half2_t{f[0], f[1]}, one, lo, false);
+                hi = __builtin_amdgcn_fdot2(half2_t{f[2], f[3]}, one, hi, false);
+                lo = __builtin_amdgcn_fdot2(half2_t{f[4], f[5]}, one, lo, false);
+                hi = __builtin_amdgcn_fdot2(half2_t{f[6], f[7]}, one, hi, false);
+            }
+            lo += __shfl_xor(lo, 16, 64);
+            hi += __shfl_xor(hi, 16, 64);
+            lo += __shfl_xor(lo, 32, 64);
+            hi += __shfl_xor(hi, 32, 64);
+            if (kq == 0) dst[r] = float2_t{ODSD_RAW_OFFSET_LO * lo + ODSD_RAW_OFFSET_HI * hi, lo + hi};
+        };
+        for (int bi = wave; bi < G_UP * MB; bi += WAVES) {
+            if (bi % MB < nmb) group_sums(xs_raw + bi * XBLK, cx + bi * 16);
+        }
+        __syncthreads();
+
         // One step = one group of one block pair: B fragments of the group from LDS, the slot's two
         // tiles expanded to fp16, the slot refilled with the step DEPTH ahead, 2 x MB x 4 MFMAs.
         // Both streams of a wavefront are unrolled: ring slots, tile offsets and LDS addresses are
         // constants, and the wait the compiler derives for a slot leaves the younger slots in flight.
         float4_t acc[2][MB];
-        auto step = [&](const int slot, const char *frag_base, auto refill) {
+        auto step = [&](const int slot, const char *frag_base, const float2_t *sums, auto refill) {
+            ODSD_FENCE();
             half8_t bx[MB][4];
+            float2_t cxv[MB];
 #pragma unroll
-            for (int m = 0; m < MB; ++m) {
-                if (m == 0 || m < nmb) {                      // (a pass has at least one row)
+            for (int m = 0; m < nmb; ++m) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) bx[m][j] = *(const half8_t *)(frag_base + m * XBLK + lds_frag[j]);
-                }
+                for (int j = 0; j < 4; ++j) bx[m][j] = *(const half8_t *)(frag_base + m * XBLK + lds_frag[j]);
+                cxv[m] = sums[m * 16 + r];
             }
             half8_t a[2][4];
 #pragma unroll
-            for (int i = 0; i < 2; ++i) dequant_tile(dc, wq[slot][i], wsz[slot][i], a[i]);
-            __builtin_amdgcn_sched_barrier(0);
+            for (int i = 0; i < 2; ++i) {
+                a[i][0] = raw_word(rc, wq[slot][i].x);
+                a[i][1] = raw_word(rc, wq[slot][i].y);
+                a[i][2] = raw_word(rc, wq[slot][i].z);
+                a[i][3] = raw_word(rc, wq[slot][i].w);
+            }
+            const uint4_t sz0 = wsz[slot][0], sz1 = wsz[slot][1];
+            ODSD_FENCE();
             refill();                                         // the slot is free again
-            __builtin_amdgcn_sched_barrier(0);
+            ODSD_FENCE();
 #pragma unroll
-            for (int m = 0; m < MB; ++m) {
-                if (m == 0 || m < nmb) {
+            for (int m = 0; m < nmb; ++m) {
+                {
+                    // the group's sum of q_k x_k: the accumulator starts at minus the offsets' share
+                    const float nc = -cxv[m].x, xsum = cxv[m].y;
+                    float4_t t[2];
+                    t[0] = t[1] = float4_t{nc, nc, nc, nc};
 #pragma unroll
                     for (int j = 0; j < 4; ++j)
 #pragma unroll
-                        for (int i = 0; i < 2; ++i) acc[i][m] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i][j], bx[m][j], acc[i][m], 0, 0, 0);
+                        for (int i = 0; i < 2; ++i)
+                            t[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i][j], bx[m][j], t[i], 0, 0, 0);
+                    // w = (q - zero) * scale per output row: acc += scale * (sum q x - zero * sum x)
+#pragma unroll
+                    for (int i = 0; i < 2; ++i) {
+                        const uint4_t sz = i ? sz1 : sz0;
+                        const half2_t p0 = as_half2(sz.x), p1 = as_half2(sz.y), p2 = as_half2(sz.z), p3 = as_half2(sz.w);
+                        acc[i][m].x = __builtin_fmaf((float)p0.x, __builtin_fmaf(-(float)p0.y, xsum, t[i].x), acc[i][m].x);
+                        acc[i][m].y = __builtin_fmaf((float)p1.x, __builtin_fmaf(-(float)p1.y, xsum, t[i].y), acc[i][m].y);
+                        acc[i][m].z = __builtin_fmaf((float)p2.x, __builtin_fmaf(-(float)p2.y, xsum, t[i].z), acc[i][m].z);
+                        acc[i][m].w = __builtin_fmaf((float)p3.x, __builtin_fmaf(-(float)p3.y, xsum, t[i].w), acc[i][m].w);
+                    }
                 }
             }
-            __builtin_amdgcn_sched_barrier(0);
+            // the step's arithmetic has no memory side: tie its results to the fence, or the whole
+            // chain of a step may be ordered behind the loads of the steps after it
+#pragma unroll
+            for (int m = 0; m < nmb; ++m)
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+                    asm volatile("" : "+v"(acc[i][m].x), "+v"(acc[i][m].y), "+v"(acc[i][m].z), "+v"(acc[i][m].w));
+            ODSD_FENCE();
         };
         auto zero_acc = [&]() {
 #pragma unroll
@@ -194,7 +300,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
         for (int t = 0; t < NT; ++t) {
             const int pi = t / G_UP, g = t % G_UP;
             if (g == 0) zero_acc();
-            step(t % DEPTH, xs_raw + (g * MB) * XBLK, [&]() {
+            step(t % DEPTH, xs_raw + (g * MB) * XBLK, cx + (g * MB) * 16, [&]() {
                 // past the end of gate_up the ring goes on with the first steps of the down stream
                 if (t + DEPTH < NT) load_u(t % DEPTH, t + DEPTH);
                 else if (t + DEPTH - NT < ntd_w) load_d(t % DEPTH, t + DEPTH - NT);
@@ -205,8 +311,8 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
                 const int fbl = wave * PPW + pi;             // 16-feature block inside the slice
                 const int gl = fbl >> 3, seg = (fbl & 7) * 2 + (kq >> 1);
 #pragma unroll
-                for (int m = 0; m < MB; ++m) {
-                    if (m == 0 || m < nmb) {
+                for (int m = 0; m < nmb; ++m) {
+                    {
                         const float4_t gt = acc[0][m], up = acc[1][m];
                         half4_t h;
                         h.x = f32_to_f16_sat(silu_f32(gt.x) * up.x);
@@ -220,6 +326,10 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
             }
         }
         __syncthreads();                                      // h is complete
+        for (int bi = wave; bi < GS * MB; bi += WAVES) {
+            if (bi % MB < nmb) group_sums(hs_raw + bi * XBLK, cx + (G_UP * MB + bi) * 16);
+        }
+        __syncthreads();
 
         // down: step u = group u % GS of output block pair u / GS, against h from LDS; the slice's
         // partial sums are stored as fp16 when a pair's last group is done
@@ -228,15 +338,15 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
             if (u >= DP_MIN * GS && u >= ntd_w) break;
             const int pi = u / GS, gl = u % GS;
             if (gl == 0) zero_acc();
-            step((NT + u) % DEPTH, hs_raw + (gl * MB) * XBLK, [&]() {
+            step((NT + u) % DEPTH, hs_raw + (gl * MB) * XBLK, cx + ((G_UP + gl) * MB) * 16, [&]() {
                 if (u + DEPTH < NTD && u + DEPTH < ntd_w) load_d((NT + u) % DEPTH, u + DEPTH);
             });
             if (gl == GS - 1) {
                 // lane holds outputs 4*kq .. 4*kq+3 of each block, token column r
 #pragma unroll
-                for (int m = 0; m < MB; ++m) {
+                for (int m = 0; m < nmb; ++m) {
                     const int row = m * 16 + r;
-                    if (m < nmb && row < mcnt) {
+                    if (row < mcnt) {
                         const size_t slot = (size_t)(base + m0 + row);
                         half_t *yrow = p.y + ((size_t)s * p.P + slot) * p.H;
 #pragma unroll
@@ -250,6 +360,9 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
                 }
             }
         }
+        };   // run_pass
+        if (MB == 1 || mcnt <= 16) run_pass(std::integral_constant<int, 1>{});
+        else run_pass(std::integral_constant<int, MB>{});
     }
 }
 
