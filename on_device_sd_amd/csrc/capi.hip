@@ -98,11 +98,18 @@ static int moe_forward_impl(const odsd_moe_shape *s, const void *x, const void *
                                 l.xn - l.router, st, fold ? row_sumsq_in : nullptr, norm_weight, eps,
                                 nullptr, nullptr);
     if (rc != ODSD_OK) return rc;
-    rc = odsd_launch_dispatch(s, idx, counts, offsets, perm, inv, slot_token, st);
-    if (rc != ODSD_OK) return rc;
+    // shapes served by the one-launch expert kernel need no dispatch kernel: its workgroups scan the
+    // expert ids themselves and leave counts / offsets / perm (inv and slot_token are not produced:
+    // nothing after the experts reads them)
+    const OdsdDispatchOut inside{counts, offsets, perm, nullptr, nullptr};
+    const bool dispatch_inside = odsd_experts_dispatch_inside(s) && odsd_aligned16(idx);
+    if (!dispatch_inside) {
+        rc = odsd_launch_dispatch(s, idx, counts, offsets, perm, inv, slot_token, st);
+        if (rc != ODSD_OK) return rc;
+    }
     return odsd_launch_experts(s, x16, table, idx, w, counts, offsets, perm, slot_token,
                                add_residual ? x : nullptr, out_f32, out_act, ws + l.experts,
-                               l.total - l.experts, st, row_sumsq_out);
+                               l.total - l.experts, st, row_sumsq_out, dispatch_inside ? &inside : nullptr);
 }
 
 extern "C" int odsd_moe_forward(const odsd_moe_shape *s, const void *x, const void *norm_weight, float eps,

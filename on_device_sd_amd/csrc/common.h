@@ -132,8 +132,12 @@ int odsd_launch_router(const odsd_moe_shape *s, const void *x, const void *gate_
 int odsd_launch_dispatch(const odsd_moe_shape *s, const int32_t *idx, int32_t *counts,
                          int32_t *offsets, int32_t *perm, int32_t *inv, int32_t *slot_token,
                          hipStream_t st);
+// dispatch_out: the dispatch arrays have NOT been filled; the expert kernel dispatches for itself and
+// leaves counts / offsets / perm there (only when odsd_experts_dispatch_inside(s) says it can)
 int odsd_launch_experts(const odsd_moe_shape *s, const void *x16, const uint64_t *table,
                         const int32_t *idx, const float *w, const int32_t *counts,
                         const int32_t *offsets, const int32_t *perm, const int32_t *slot_token,
                         const void *residual, float *out_f32, void *out_act, void *ws,
-                        size_t ws_bytes, hipStream_t st, double *row_ss);
+                        size_t ws_bytes, hipStream_t st, double *row_ss,
+                        const OdsdDispatchOut *dispatch_out = nullptr);
+int odsd_experts_dispatch_inside(const odsd_moe_shape *s);

@@ -516,6 +516,7 @@ struct ExpertsPlan {
 // one-launch expert kernel (experts_fused.hip)
 void odsd_launch_experts_fused(FusedParams &fp, int E, hipStream_t st);
 int odsd_fused_supported(int H, int I, int S);
+int odsd_fused_dispatch_supported(int P);
 
 // Choices are functions of the shape only (the per-expert counts live on the device).
 static ExpertsPlan experts_plan(const odsd_moe_shape *s) {
@@ -763,7 +764,8 @@ extern "C" int odsd_combine(const odsd_moe_shape *s, const void *y, const int32_
 int odsd_launch_experts(const odsd_moe_shape *s, const void *x16, const uint64_t *table, const int32_t *idx,
                         const float *w, const int32_t *counts, const int32_t *offsets, const int32_t *perm,
                         const int32_t *slot_token, const void *residual, float *out_f32, void *out_act,
-                        void *ws, size_t ws_bytes, hipStream_t st, double *row_ss) {
+                        void *ws, size_t ws_bytes, hipStream_t st, double *row_ss,
+                        const OdsdDispatchOut *dispatch_out) {
     int rc = experts_check(s);
     if (rc != ODSD_OK) return rc;
     if (s->T == 0) return ODSD_OK;
@@ -773,14 +775,22 @@ int odsd_launch_experts(const odsd_moe_shape *s, const void *x16, const uint64_t
     if (ws_bytes < pl.h_bytes + pl.y_bytes) return ODSD_ERR_WORKSPACE;
     void *h16 = ws;
     float *y = (float *)((char *)ws + pl.h_bytes);
+    if (dispatch_out && !(pl.fused && odsd_fused_dispatch_supported(s->T * s->K))) return ODSD_ERR_UNSUPPORTED;
     if (pl.fused) {
-        if (!x16 || !table || !counts || !offsets || !slot_token) return ODSD_ERR_NULL;
+        if (!x16 || !table || !counts || !offsets || (!slot_token && !dispatch_out)) return ODSD_ERR_NULL;
         if (!odsd_aligned16(x16)) return ODSD_ERR_ALIGN;
         FusedParams fp{};
         fp.table = table; fp.x16 = (const half_t *)x16; fp.rowmap = slot_token;
         fp.counts = counts; fp.offsets = offsets; fp.y = (half_t *)y;
         fp.H = s->H; fp.I = s->I; fp.S = pl.S; fp.P = s->T * s->K;
         fp.G_up = s->H / ODSD_GROUP; fp.G_dn = s->I / ODSD_GROUP;
+        fp.K = s->K; fp.E = s->E;
+        if (dispatch_out) {
+            if (!idx || !dispatch_out->counts || !dispatch_out->offsets || !dispatch_out->perm) return ODSD_ERR_NULL;
+            if (!odsd_aligned16(idx)) return ODSD_ERR_ALIGN;
+            fp.idx = idx;
+            fp.out_counts = dispatch_out->counts; fp.out_offsets = dispatch_out->offsets; fp.out_perm = dispatch_out->perm;
+        }
         odsd_launch_experts_fused(fp, s->E, st);
         ODSD_CHECK_LAUNCH();
         return launch_combine(s, y, idx, w, perm, table, residual, out_f32, out_act, row_ss, st, pl.S);
@@ -790,6 +800,14 @@ int odsd_launch_experts(const odsd_moe_shape *s, const void *x16, const uint64_t
     rc = odsd_w4_down(s, h16, table, counts, offsets, y, st);
     if (rc != ODSD_OK) return rc;
     return launch_combine(s, y, idx, w, perm, table, residual, out_f32, out_act, row_ss, st);
+}
+
+// 1: a whole-block call may skip the dispatch kernel for this shape (the expert kernel scans the
+// expert ids itself)
+int odsd_experts_dispatch_inside(const odsd_moe_shape *s) {
+    if (experts_check(s) != ODSD_OK) return 0;
+    const ExpertsPlan pl = experts_plan(s);
+    return pl.fused && odsd_fused_dispatch_supported(s->T * s->K);
 }
 
 extern "C" int odsd_experts_w4(const odsd_moe_shape *s, const void *x_f16, const uint64_t *table,

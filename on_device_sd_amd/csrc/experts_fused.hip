@@ -76,7 +76,12 @@ typedef float float2_t __attribute__((ext_vector_type(2)));
 // WAVES wavefronts per workgroup
 // G_UP  H / 128, G_DN  I / 128: groups of the two reductions (compile time: every tile offset of
 //       a wavefront's stream is a constant)
-template <int MB, int GS, int WAVES, int G_UP, int G_DN>
+// DISP  the workgroup dispatches for itself: it scans the [P] expert ids (P <= 4 * 64 * WAVES, one
+//       vector of 4 per thread), counts the pairs of its expert and of lower experts (ballot /
+//       popcount, the order of the pair list is kept: stable), keeps its expert's token rows in LDS
+//       and, as slice 0, writes counts[e], offsets[e] and the slots of its pairs -- what the
+//       separate dispatch kernel and two dependent loads per workgroup did before
+template <int MB, int GS, int WAVES, int G_UP, int G_DN, bool DISP>
 __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(const FusedParams p) {
     static_assert(WAVES % 4 == 0 && (8 * GS) % WAVES == 0, "whole gate/up block pairs per wavefront");
     static_assert(G_UP * MB <= ODSD_FUSED_X_BLOCKS, "token rows of a pass must fit the LDS area");
@@ -94,14 +99,71 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
     // per (group, token block) and token row: (sum of offset_k * x_k, sum of x_k) over the group's 128
     // columns -- the token rows' blocks first, the blocks of h after them
     __shared__ float2_t cx[(G_UP + GS) * MB * 16];
+    __shared__ int32_t rows_lds[16 * MB];        // DISP: tokens of the pass's rows
+    __shared__ int32_t wsum[2][WAVES];           // DISP: per-wavefront totals (pairs of e, pairs below e)
 
     const int b = blockIdx.x;
     const int e = b / p.S, s = b - e * p.S;
     // everything the prologue depends on is requested at once (one round trip, not three)
     const uint64_t *trow = p.table + (size_t)e * ODSD_TABLE_COLS;
-    const int M_e = p.counts[e];
-    const int base = p.offsets[e];
     const uint64_t t_gu_q = trow[0], t_gu_sz = trow[1], t_dn_q = trow[2], t_dn_sz = trow[3];
+    int M_e, base;
+    int rk[4] = {-1, -1, -1, -1};                // DISP: rank of this thread's pairs inside the expert, or -1
+    int pair0 = 0;
+    if (DISP) {
+        const int tid_ = threadIdx.x, lane_ = tid_ & 63, wave_ = tid_ >> 6;
+        pair0 = 4 * tid_;
+        int id[4] = {-1, -1, -1, -1};
+        if (pair0 < p.P) {                       // P is a multiple of 4
+            const uint4_t v = *(const uint4_t *)(p.idx + pair0);
+            id[0] = (int)v.x; id[1] = (int)v.y; id[2] = (int)v.z; id[3] = (int)v.w;
+        }
+        int cm = 0, cl = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            cm += id[j] == e;
+            cl += (uint32_t)id[j] < (uint32_t)e; // ids outside [0, E) belong to nobody
+        }
+        // counts of at most 4 per lane: three ballots give the prefix over the lower lanes and the total
+        const uint64_t m0b = __ballot(cm & 1), m1b = __ballot(cm & 2), m2b = __ballot(cm & 4);
+        const uint64_t l0b = __ballot(cl & 1), l1b = __ballot(cl & 2), l2b = __ballot(cl & 4);
+        const int pre = mask_rank(m0b) + 2 * mask_rank(m1b) + 4 * mask_rank(m2b);
+        if (lane_ == 0) {
+            wsum[0][wave_] = __popcll(m0b) + 2 * __popcll(m1b) + 4 * __popcll(m2b);
+            wsum[1][wave_] = __popcll(l0b) + 2 * __popcll(l1b) + 4 * __popcll(l2b);
+        }
+        __syncthreads();
+        int before = 0, tot_m = 0, tot_l = 0;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) {
+            const int a = wsum[0][w];
+            if (w < wave_) before += a;
+            tot_m += a;
+            tot_l += wsum[1][w];
+        }
+        M_e = tot_m;
+        base = tot_l;
+        int rank = before + pre;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (id[j] == e) rk[j] = rank++;
+        }
+        if (s == 0) {
+            if (tid_ == 0) {
+                p.out_counts[e] = M_e;
+                p.out_offsets[e] = base;
+                if (e == p.E - 1) p.out_offsets[p.E] = base + M_e;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                // (the ids come from this library's router, so every pair belongs to some expert's workgroup)
+                if (rk[j] >= 0) p.out_perm[pair0 + j] = base + rk[j];
+            }
+        }
+    } else {
+        M_e = p.counts[e];
+        base = p.offsets[e];
+    }
     if (M_e == 0 || t_gu_q == 0) return;
     const global_char *src_c = (const global_char *)p.x16;
     // the expert's packed matrices and their (scale, zero) pairs as buffer resources (reads past
@@ -156,6 +218,14 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
 
     for (int m0 = 0; m0 < M_e; m0 += 16 * MB) {
         const int mcnt = min(M_e - m0, 16 * MB);
+        if (DISP) {
+            // tokens of this pass's rows (readers of the previous pass's list passed several barriers ago)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int rel = rk[j] - m0;
+                if (rk[j] >= 0 && rel >= 0 && rel < 16 * MB) rows_lds[rel] = (pair0 + j) / p.K;
+            }
+        }
         __syncthreads();                                      // the previous pass is done with both LDS areas
         // The pass is compiled once per number of token blocks that hold rows: with a run-time count
         // the values that exist on one path only (fragments, group sums, the second block's partial
@@ -191,7 +261,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
         {
             const int row = dm * 16 + row_in_blk;
             const int slot = base + m0 + (row < mcnt ? row : 0);
-            const int srow = p.rowmap[slot];
+            const int srow = DISP ? rows_lds[row < mcnt ? row : 0] : p.rowmap[slot];
             const uint32_t st_off = ((uint32_t)srow * (uint32_t)p.H + (uint32_t)((r ^ row_in_blk) * 8)) * 2u;
             if (dm < nmb && wave < 8) {
                 for (int i = 0; i < N_PIECES; ++i) {
@@ -369,8 +439,14 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
 // Shapes the fused kernel is built for; the caller has checked them with odsd_fused_supported().
 void odsd_launch_experts_fused(FusedParams &fp, int E, hipStream_t st) {
     // (MB = 2: up to 32 rows per pass; experts with at most 16 rows skip the second token block)
-    ODSD_LAUNCH(ODSD_KERNEL_EXPERTS, (w4_expert_fused_kernel<2, 3, 8, 16, 6>), E * fp.S, 512, st, fp);
+    if (fp.idx)
+        ODSD_LAUNCH(ODSD_KERNEL_EXPERTS, (w4_expert_fused_kernel<2, 3, 8, 16, 6, true>), E * fp.S, 512, st, fp);
+    else
+        ODSD_LAUNCH(ODSD_KERNEL_EXPERTS, (w4_expert_fused_kernel<2, 3, 8, 16, 6, false>), E * fp.S, 512, st, fp);
 }
+
+// the in-kernel dispatch holds the whole id list in one vector of 4 ids per thread
+int odsd_fused_dispatch_supported(int P) { return P % 4 == 0 && P <= 4 * 512; }
 
 // H = 2048 (4 sub-passes of 8 wavefronts x 4 blocks), slices of 384 features, token rows of one
 // pass within the 128 KB row area

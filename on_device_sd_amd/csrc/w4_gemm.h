@@ -44,6 +44,11 @@ struct FusedParams {
     int S;                   // slices of the intermediate dimension (workgroups per expert)
     int P;
     int G_up, G_dn;          // H / 128, I / 128
+    // dispatch inside the kernel (idx given): every workgroup finds its expert's pairs in the id
+    // list itself, and slice 0 of each expert leaves counts / offsets / perm for the combine
+    const int32_t *idx;      // [P] expert id per (token, k) pair, or null: counts / offsets / rowmap are inputs
+    int32_t *out_counts, *out_offsets, *out_perm;
+    int K, E;
 };
 
 __device__ __forceinline__ half2_t as_half2(uint32_t u) { return __builtin_bit_cast(half2_t, u); }

@@ -106,3 +106,29 @@ def test_fused_experts_vs_stages_and_oracle(dev, layer, T, forced):
     # a second run gives the same bits
     out32b, _ = ops.experts_w4(x16, bank.table(), idx, w, disp, I, torch.bfloat16, want_f32=True, want_act=False)
     assert torch.equal(out32b, out32)
+
+
+@pytest.mark.parametrize("T", [256, 136])
+def test_whole_block_dispatches_inside_the_expert_kernel(dev, layer, T):
+    """odsd_moe_forward at this shape launches no dispatch kernel: the expert kernel's workgroups
+    scan the expert ids themselves.  Indices, counts, offsets and the permutation must still be
+    the oracle's, bit for bit, and the output within tolerance."""
+    print("fused experts, dispatch inside", T, flush=True)
+    from on_device_sd_amd import ops
+    bank, experts = layer
+    g = torch.Generator().manual_seed(1000 + T)
+    wg = (torch.randn(E, H, generator=g) * 0.02).to(torch.bfloat16)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    out = ops.moe_forward(x.to(dev), wg.to(dev), bank.table(), K, I, renorm=True)
+    torch.cuda.synchronize()
+    ref, idx, w = orc.moe_block(x, wg, experts, K, True)
+    assert np.array_equal(out.idx.cpu().numpy(), idx)
+    c, o, perm, _ = orc.dispatch(idx, E)
+    assert np.array_equal(out.counts.cpu().numpy(), c)
+    assert np.array_equal(out.offsets.cpu().numpy(), o)
+    assert np.array_equal(out.perm.cpu().numpy(), perm)
+    mx, mean = check_output(out.out_f32, ref)
+    check_output_relative(out.out_f32, ref)
+    print(f"  vs oracle: max-abs {mx:.3e} mean-abs {mean:.3e}", flush=True)
+    out2 = ops.moe_forward(x.to(dev), wg.to(dev), bank.table(), K, I, renorm=True)
+    assert torch.equal(out2.out_f32, out.out_f32) and torch.equal(out2.perm, out.perm)
