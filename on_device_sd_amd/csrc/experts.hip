@@ -67,22 +67,25 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
     const int chunk = (L / p.KS) % p.nchunks;
     const int e = L / (p.KS * p.nchunks);
 
-    const int M_e = p.counts[e];
-    if (M_e == 0) return;
+    // the row count, the table row and the first slot are requested together: one round trip to
+    // memory before the first weight load instead of three dependent ones
     const uint64_t *trow = p.table + (size_t)e * ODSD_TABLE_COLS;
-    if (trow[0] == 0) return;
+    const int M_e = p.counts[e];
+    const int base = p.offsets[e];
+    const uint64_t t_present = trow[0];
+    const uint64_t t_q = MODE == 0 ? trow[0] : trow[2], t_sz = MODE == 0 ? trow[1] : trow[3];
+    if (M_e == 0 || t_present == 0) return;
     // addresses from the table are global memory: say so, or the loads become flat loads
     // whose LDS-side counter forces every wait to drain
-    const global_char *qp_c = (const global_char *)(MODE == 0 ? trow[0] : trow[2]);
-    const global_char *szp_c = (const global_char *)(MODE == 0 ? trow[1] : trow[3]);
+    const global_char *qp_c = (const global_char *)t_q;
+    const global_char *szp_c = (const global_char *)t_sz;
     const global_char *src_c = (const global_char *)p.src;
-    const int base = p.offsets[e];
     // the expert's packed matrix and its (scale, zero) pairs as buffer resources (reads past the
     // end return zero)
     const __amdgpu_buffer_rsrc_t rsrc_q = __builtin_amdgcn_make_buffer_rsrc(
-        (void *)(uintptr_t)(MODE == 0 ? trow[0] : trow[2]), 0, p.NBLK * p.G * 1024, 0x00020000);
+        (void *)(uintptr_t)t_q, 0, p.NBLK * p.G * 1024, 0x00020000);
     const __amdgpu_buffer_rsrc_t rsrc_sz = __builtin_amdgcn_make_buffer_rsrc(
-        (void *)(uintptr_t)(MODE == 0 ? trow[1] : trow[3]), 0, p.NBLK * p.G * 64, 0x00020000);
+        (void *)(uintptr_t)t_sz, 0, p.NBLK * p.G * 64, 0x00020000);
 
     const DequantConsts dc = dequant_consts();
     const int tid = threadIdx.x;
@@ -369,7 +372,7 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
 // and weight first, then KB independent row loads -- and added in k order; with the generic loop
 // every row load waits for the one before it (its address hangs on a branch), which is what the
 // kernel's time consists of at K = 8.
-// YH: 0 = y holds fp32 partial sums; 1 = fp16 values in KS slices; 2 = exactly two fp16 slices
+// YH: 0 = y holds fp32 partial sums of KS slices; 1 = complete sums as fp16; 2 = two fp16 slices
 template <typename XT, int YH, bool STATS, int KB>
 __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ y, const int32_t *__restrict__ idx,
                                                       const float *__restrict__ w,
@@ -425,11 +428,6 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
                     if (YH) {
                         const half4_t hv = *(const half4_t *)((const half_t *)y + (size_t)slot[u] * H + c);
                         v[u] = float4_t{(float)hv.x, (float)hv.y, (float)hv.z, (float)hv.w};
-                        // fp16 partial sums of further slices of the reduction, added in slice order
-                        for (int s = 1; s < KS; ++s) {
-                            const half4_t hs = *(const half4_t *)((const half_t *)y + ((size_t)s * P + slot[u]) * H + c);
-                            v[u] += float4_t{(float)hs.x, (float)hs.y, (float)hs.z, (float)hs.w};
-                        }
                     } else {
                         v[u] = *(const float4_t *)(y + (size_t)slot[u] * H + c);
                     }
@@ -453,11 +451,11 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
             if (slot < 0 || e < 0 || e >= E || table[(size_t)e * ODSD_TABLE_COLS] == 0) continue;
             float4_t v;
             if (YH) {
-                // fp16 values: complete sums (KS == 1) or the partial sums of KS slices
+                // fp16 values: complete sums (YH == 1) or the partial sums of two slices (YH == 2)
                 const half4_t hv = *(const half4_t *)((const half_t *)y + (size_t)slot * H + c);
                 v = float4_t{(float)hv.x, (float)hv.y, (float)hv.z, (float)hv.w};
-                for (int s = 1; s < KS; ++s) {
-                    const half4_t hs = *(const half4_t *)((const half_t *)y + ((size_t)s * P + slot) * H + c);
+                if (YH == 2) {
+                    const half4_t hs = *(const half4_t *)((const half_t *)y + ((size_t)P + slot) * H + c);
                     v += float4_t{(float)hs.x, (float)hs.y, (float)hs.z, (float)hs.w};
                 }
             } else {
@@ -590,7 +588,7 @@ static ExpertsPlan experts_plan(const odsd_moe_shape *s) {
     p.S = 1;
     if (p.MB == 2 && s->T > 16 && mean_rows >= 8) {
         int S = 256 / s->E;
-        if (S >= 1 && S <= 4 && s->E * S >= 192 && odsd_fused_supported(s->H, s->I, S)) {
+        if (S >= 1 && S <= 2 && s->E * S >= 192 && odsd_fused_supported(s->H, s->I, S)) {
             p.fused = 1;
             p.S = S;
             const size_t need = odsd_round_up((size_t)S * (size_t)P * s->H * sizeof(half_t), 256);
@@ -719,6 +717,7 @@ static int launch_combine(const odsd_moe_shape *s, const void *y_, const int32_t
     if (row_ss && !out_act) return ODSD_ERR_NULL;
     if (!odsd_aligned16(y) || (out_f32 && !odsd_aligned16(out_f32))) return ODSD_ERR_ALIGN;
     ExpertsPlan pl = experts_plan(s);
+    if (y_slices > 2) return ODSD_ERR_UNSUPPORTED;          // fp16 partial sums: one or two slices
     if (y_slices > 0) { pl.KS = y_slices; pl.y_f16 = 1; }
     const int P = s->T * s->K;
     const int nchunk = (s->H / 4 + 255) / 256;

@@ -47,14 +47,16 @@ __global__ __launch_bounds__(512, 2) void w4_gemm_prefill_kernel(const GemmParam
     const int ps = (L / (p.nchunks * p.KS)) % p.PS;
     const int e = L / (p.nchunks * p.KS * p.PS);
 
-    const int M_e = p.counts[e];
-    if (M_e == 0) return;
+    // requested together: one round trip to memory instead of three dependent ones
     const uint64_t *trow = p.table + (size_t)e * ODSD_TABLE_COLS;
-    if (trow[0] == 0) return;
-    const global_char *qp_c = (const global_char *)(MODE == 0 ? trow[0] : trow[2]);
-    const global_char *szp_c = (const global_char *)(MODE == 0 ? trow[1] : trow[3]);
-    const global_char *src_c = (const global_char *)p.src;
+    const int M_e = p.counts[e];
     const int base = p.offsets[e];
+    const uint64_t t_present = trow[0];
+    const uint64_t t_q = MODE == 0 ? trow[0] : trow[2], t_sz = MODE == 0 ? trow[1] : trow[3];
+    if (M_e == 0 || t_present == 0) return;
+    const global_char *qp_c = (const global_char *)t_q;
+    const global_char *szp_c = (const global_char *)t_sz;
+    const global_char *src_c = (const global_char *)p.src;
     // gate_up reads its weights through buffer loads: resource in scalar registers, constant
     // per-lane offset, the group as the scalar offset -- no vector instruction per address
     const __amdgpu_buffer_rsrc_t rsrc_q = __builtin_amdgcn_make_buffer_rsrc((void *)(uintptr_t)qp_c, 0, p.NBLK * p.G * 1024, 0x00020000);
