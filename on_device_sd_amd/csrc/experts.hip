@@ -581,12 +581,14 @@ static ExpertsPlan experts_plan(const odsd_moe_shape *s) {
     p.h_bytes = odsd_round_up((size_t)(P > 0 ? P : 1) * s->I * sizeof(half_t), 256);
     p.y_bytes = odsd_round_up((size_t)p.KS * (size_t)(P > 0 ? P : 1) * s->H * sizeof(float), 256);
     // The one-launch expert kernel serves calls where nearly every expert has rows and a pass holds
-    // them all (8 to 16 rows per expert on average, at most 32 per pass): one workgroup per
+    // them all (8 to 20 rows per expert on average, at most 32 per pass; measured against the
+    // two-launch plan on uniform routing it wins up to 20 and loses from 24 on, where many experts
+    // need a second pass over their weights): one workgroup per
     // (expert, slice of the intermediate dimension), E * S workgroups for 256 CUs.  The stage entry
     // points keep the two-launch plan above; only the whole-block calls take this path.
     p.fused = 0;
     p.S = 1;
-    if (p.MB == 2 && s->T > 16 && mean_rows >= 8) {
+    if (s->T > 16 && mean_rows >= 8 && mean_rows <= 20) {
         int S = 256 / s->E;
         if (S >= 1 && S <= 2 && s->E * S >= 192 && odsd_fused_supported(s->H, s->I, S)) {
             p.fused = 1;

@@ -1,7 +1,7 @@
 """The one-launch expert kernel (gate_up -> SiLU*mul -> down in one workgroup per expert slice).
 
 It serves whole-block calls at the Qwen3-30B-A3B expert shape (hidden 2048, 128 experts, top 8,
-intermediate 768) with 8 to 16 rows per expert on average; the stage entry points keep the
+intermediate 768) with 8 to 20 rows per expert on average; the stage entry points keep the
 two-launch plan.  The same hand-built routing goes through both, and through the CPU oracle:
 experts without rows, with exactly 16 / 17 / 32 / 33 rows (one and two token blocks, one and two
 passes) and one with 70 rows (three passes).  Replaces expert_forward_with_weights
@@ -58,6 +58,7 @@ CASES = [
     # T, {expert: rows}
     (256, {}),                                                   # the benchmark's shape, uniform routing
     (128, {}),                                                   # 8 rows per expert on average
+    (320, {}),                                                   # 20 on average: some experts take two passes
     (200, {0: 0, 1: 16, 2: 17, 3: 32, 4: 33, 5: 70, 6: 1, 127: 0}),
 ]
 
