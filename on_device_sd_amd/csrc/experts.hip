@@ -34,8 +34,13 @@
 //       (global_load_lds, no registers), double buffered, 16-byte segments XOR-swizzled
 //       by the row so that the B-fragment reads are bank-conflict free; one raw s_barrier
 //       per group, preceded by a vmcnt wait that leaves the newest loads in flight.
-template <int NB, int MB, int MODE, int DEPTH, int NA, int WK, bool DIRECT, int OCC, int WAVES>
+// DISP  (gate_up only) the workgroup dispatches for itself: it scans the [P] expert ids (P <= 4
+//       per thread), counts the pairs of its expert and of lower experts (ballot / popcount; the
+//       order of the pair list is kept: stable), keeps the tokens of a pass's rows in LDS, and the
+//       first workgroup of each expert writes counts[e], offsets[e] and the slots of its pairs
+template <int NB, int MB, int MODE, int DEPTH, int NA, int WK, bool DIRECT, int OCC, int WAVES, bool DISP>
 __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmParams p) {
+    static_assert(!DISP || MODE == 0, "only gate_up dispatches");
     static_assert(MODE == 1 || NB % 2 == 0, "gate_up needs gate/up block pairs");
     static_assert(NB % NA == 0, "NA must divide NB");
     static_assert(!DIRECT || MB == 1, "the direct path holds one token block");
@@ -54,6 +59,8 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
     constexpr int LDS_BYTES = DIRECT ? (WK > 1 ? RED_FLOATS * 4 : 16) : XS_BYTES;
     __shared__ __attribute__((aligned(16))) char xs_raw[LDS_BYTES];
     float *red = (float *)xs_raw;
+    __shared__ int32_t rows_lds[DISP ? 16 * MB : 1];    // DISP: tokens of the pass's rows
+    __shared__ int32_t wsum[2][DISP ? WAVES : 1];        // DISP: per-wavefront totals (pairs of e, pairs below e)
 
     // workgroup -> (expert, row chunk, k split).  Hardware deals workgroups round-robin over
     // the 8 XCDs.  With many token rows per expert (MB >= 6) consecutive logical ids are kept
@@ -70,10 +77,75 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
     // the row count, the table row and the first slot are requested together: one round trip to
     // memory before the first weight load instead of three dependent ones
     const uint64_t *trow = p.table + (size_t)e * ODSD_TABLE_COLS;
-    const int M_e = p.counts[e];
-    const int base = p.offsets[e];
     const uint64_t t_present = trow[0];
     const uint64_t t_q = MODE == 0 ? trow[0] : trow[2], t_sz = MODE == 0 ? trow[1] : trow[3];
+    int M_e, base;
+    // DISP: one scan of the id list gives the expert's row count, its first slot and -- for the rows
+    // m0 .. m0 + 16 MB - 1 of the expert -- their tokens (in LDS).  Nothing of it is kept in registers:
+    // a further pass scans again.
+    auto scan_rows = [&](const int m0, const bool first) {
+        const int tid_ = threadIdx.x, lane_ = tid_ & 63, wave_ = tid_ >> 6;
+        const int pair0 = 4 * tid_;
+        int id[4] = {-1, -1, -1, -1};
+        if (pair0 + 3 < p.P) {
+            const uint4_t v = *(const uint4_t *)(p.idx + pair0);
+            id[0] = (int)v.x; id[1] = (int)v.y; id[2] = (int)v.z; id[3] = (int)v.w;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (pair0 + j < p.P) id[j] = p.idx[pair0 + j];   // the list's ragged end
+        }
+        int cm = 0, cl = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            cm += id[j] == e;
+            cl += (uint32_t)id[j] < (uint32_t)e; // ids outside [0, E) belong to nobody
+        }
+        // counts of at most 4 per lane: three ballots give the prefix over the lower lanes and the total
+        const uint64_t m0b = __ballot(cm & 1), m1b = __ballot(cm & 2), m2b = __ballot(cm & 4);
+        const uint64_t l0b = __ballot(cl & 1), l1b = __ballot(cl & 2), l2b = __ballot(cl & 4);
+        const int pre = mask_rank(m0b) + 2 * mask_rank(m1b) + 4 * mask_rank(m2b);
+        __syncthreads();                          // the previous scan's totals and row list have been read
+        if (lane_ == 0) {
+            wsum[0][wave_] = __popcll(m0b) + 2 * __popcll(m1b) + 4 * __popcll(m2b);
+            wsum[1][wave_] = __popcll(l0b) + 2 * __popcll(l1b) + 4 * __popcll(l2b);
+        }
+        __syncthreads();
+        int before = 0, tot_m = 0, tot_l = 0;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) {
+            const int a = wsum[0][w];
+            if (w < wave_) before += a;
+            tot_m += a;
+            tot_l += wsum[1][w];
+        }
+        M_e = tot_m;
+        base = tot_l;
+        int rank = before + pre;
+        const bool writer = first && chunk == 0 && ks == 0;
+        if (writer && tid_ == 0) {
+            p.out_counts[e] = tot_m;
+            p.out_offsets[e] = tot_l;
+            if (e == p.E - 1) p.out_offsets[p.E] = tot_l + tot_m;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (id[j] == e) {
+                const int rel = rank - m0;
+                if (rel >= 0 && rel < 16 * MB) rows_lds[rel] = (pair0 + j) / p.K;
+                // (the ids come from this library's router, so every pair belongs to some expert's workgroup)
+                if (writer) p.out_perm[pair0 + j] = tot_l + rank;
+                ++rank;
+            }
+        }
+        __syncthreads();                          // the row list is complete
+    };
+    if (DISP) {
+        scan_rows(0, true);
+    } else {
+        M_e = p.counts[e];
+        base = p.offsets[e];
+    }
     if (M_e == 0 || t_present == 0) return;
     // addresses from the table are global memory: say so, or the loads become flat loads
     // whose LDS-side counter forces every wait to drain
@@ -130,6 +202,7 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
         const int mcnt = min(M_e - m0, 16 * MB);
         const int nmb = (mcnt + 15) >> 4;
         const int mcnt_s = DIRECT ? mcnt : scalar_int(mcnt);
+        if (DISP && m0 > 0) scan_rows(m0, false);   // the tokens of this pass's rows
 
         // byte offsets of the token rows this thread fetches
         //   DMA path:    piece i -> row st_row0 + 16 i, source segment st_seg ^ (row & 15)
@@ -141,7 +214,7 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
         for (int i = 0; i < XPT; ++i) {
             const int row = DIRECT ? r : st_row0 + ROWS_PER_PIECE * i;
             const int slot = base + m0 + (row < mcnt ? row : 0);
-            const int srow = p.rowmap ? p.rowmap[slot] : slot;
+            const int srow = DISP ? rows_lds[row < mcnt ? row : 0] : (p.rowmap ? p.rowmap[slot] : slot);
             const int seg = DIRECT ? kq : (st_seg ^ (row & 15));
             st_off[i] = ((uint32_t)srow * (uint32_t)p.src_ld + seg * 8) * 2u;
         }
@@ -627,8 +700,15 @@ static void launch_gemm(GemmParams &gp, hipStream_t st) {
     gp.nchunks = (gp.NBLK + (WAVES / WK) * NB - 1) / ((WAVES / WK) * NB);
     gp.n_wg = gp.E * gp.nchunks * gp.KS;
     gp.wg_per_xcd = (gp.n_wg + 7) / 8;
+    if constexpr (MODE == 0 && MB == 2) {
+        if (gp.idx) {
+            ODSD_LAUNCH(ODSD_KERNEL_GATE_UP, (w4_gemm_kernel<NB, MB, MODE, DEPTH, NA, WK, DIRECT, OCC, WAVES, true>),
+                        gp.wg_per_xcd * 8, 64 * WAVES, st, gp);
+            return;
+        }
+    }
     ODSD_LAUNCH(MODE == 0 ? ODSD_KERNEL_GATE_UP : ODSD_KERNEL_DOWN,
-                (w4_gemm_kernel<NB, MB, MODE, DEPTH, NA, WK, DIRECT, OCC, WAVES>), gp.wg_per_xcd * 8, 64 * WAVES, st, gp);
+                (w4_gemm_kernel<NB, MB, MODE, DEPTH, NA, WK, DIRECT, OCC, WAVES, false>), gp.wg_per_xcd * 8, 64 * WAVES, st, gp);
 }
 
 // prefill-shaped tile kernel (experts_prefill.hip)
@@ -661,13 +741,25 @@ static int experts_args_ok(const odsd_moe_shape *s) {
 }
 
 // gate_up + SiLU*mul: x_f16 [T,H] gathered by slot_token -> h_f16 [P,I] in slot order
-extern "C" int odsd_w4_gate_up_silu(const odsd_moe_shape *s, const void *x_f16, const uint64_t *table,
-                                    const int32_t *counts, const int32_t *offsets,
-                                    const int32_t *slot_token, void *h_f16, void *stream) {
+// the streaming gate_up kernels scan up to 4 ids per thread of their 256
+// (measured: with 32-row passes -- many experts, a dozen workgroups each -- the scan costs the
+// gate_up kernel nothing and saves the dispatch launch, 4 us of the Zipf-skewed T = 64 layer's 81;
+// with hundreds of workgroups per expert it costs gate_up more than the launch it saves: +7 us at
+// the Mixtral T = 160 shape, +6 us at T = 5, so those plans keep the dispatch kernel)
+static bool stream_dispatch_supported(const ExpertsPlan &pl, int P) {
+    return !pl.tile && pl.MB == 2 && P <= 4 * 256;
+}
+
+// idx + dispatch_out: the dispatch arrays have not been filled; the kernel dispatches for itself
+// and leaves counts / offsets / perm in dispatch_out
+static int launch_gate_up(const odsd_moe_shape *s, const void *x_f16, const uint64_t *table,
+                          const int32_t *counts, const int32_t *offsets, const int32_t *slot_token,
+                          void *h_f16, hipStream_t st, const int32_t *idx, const OdsdDispatchOut *dispatch_out) {
     const int rc = experts_args_ok(s);
     if (rc != ODSD_OK) return rc;
     if (s->T == 0) return ODSD_OK;
-    if (!x_f16 || !table || !counts || !offsets || !slot_token || !h_f16) return ODSD_ERR_NULL;
+    if (!x_f16 || !table || !h_f16) return ODSD_ERR_NULL;
+    if (!dispatch_out && (!counts || !offsets || !slot_token)) return ODSD_ERR_NULL;
     if (!odsd_aligned16(x_f16) || !odsd_aligned16(h_f16)) return ODSD_ERR_ALIGN;
     const ExpertsPlan pl = experts_plan(s);
     GemmParams gu{};
@@ -675,9 +767,23 @@ extern "C" int odsd_w4_gate_up_silu(const odsd_moe_shape *s, const void *x_f16, 
     gu.counts = counts; gu.offsets = offsets; gu.h16 = (half_t *)h_f16; gu.y = nullptr;
     gu.src_ld = s->H; gu.G = s->H / ODSD_GROUP; gu.NBLK = 2 * s->I / 16;
     gu.KS = 1; gu.gper = gu.G; gu.PS = pl.PS_gu; gu.ldo = s->I; gu.P = s->T * s->K; gu.E = s->E;
-    launch_gemm_plan<0>(pl, gu, (hipStream_t)stream);
+    gu.K = s->K;
+    if (dispatch_out) {
+        if (!stream_dispatch_supported(pl, gu.P)) return ODSD_ERR_UNSUPPORTED;
+        if (!idx || !dispatch_out->counts || !dispatch_out->offsets || !dispatch_out->perm) return ODSD_ERR_NULL;
+        if (!odsd_aligned16(idx)) return ODSD_ERR_ALIGN;
+        gu.idx = idx;
+        gu.out_counts = dispatch_out->counts; gu.out_offsets = dispatch_out->offsets; gu.out_perm = dispatch_out->perm;
+    }
+    launch_gemm_plan<0>(pl, gu, st);
     ODSD_CHECK_LAUNCH();
     return ODSD_OK;
+}
+
+extern "C" int odsd_w4_gate_up_silu(const odsd_moe_shape *s, const void *x_f16, const uint64_t *table,
+                                    const int32_t *counts, const int32_t *offsets,
+                                    const int32_t *slot_token, void *h_f16, void *stream) {
+    return launch_gate_up(s, x_f16, table, counts, offsets, slot_token, h_f16, (hipStream_t)stream, nullptr, nullptr);
 }
 
 extern "C" int32_t odsd_w4_down_splits(const odsd_moe_shape *s) {
@@ -776,7 +882,8 @@ int odsd_launch_experts(const odsd_moe_shape *s, const void *x16, const uint64_t
     if (ws_bytes < pl.h_bytes + pl.y_bytes) return ODSD_ERR_WORKSPACE;
     void *h16 = ws;
     float *y = (float *)((char *)ws + pl.h_bytes);
-    if (dispatch_out && !(pl.fused && odsd_fused_dispatch_supported(s->T * s->K))) return ODSD_ERR_UNSUPPORTED;
+    if (dispatch_out && !(pl.fused ? odsd_fused_dispatch_supported(s->T * s->K) : stream_dispatch_supported(pl, s->T * s->K)))
+        return ODSD_ERR_UNSUPPORTED;
     if (pl.fused) {
         if (!x16 || !table || !counts || !offsets || (!slot_token && !dispatch_out)) return ODSD_ERR_NULL;
         if (!odsd_aligned16(x16)) return ODSD_ERR_ALIGN;
@@ -796,7 +903,7 @@ int odsd_launch_experts(const odsd_moe_shape *s, const void *x16, const uint64_t
         ODSD_CHECK_LAUNCH();
         return launch_combine(s, y, idx, w, perm, table, residual, out_f32, out_act, row_ss, st, pl.S);
     }
-    rc = odsd_w4_gate_up_silu(s, x16, table, counts, offsets, slot_token, h16, st);
+    rc = launch_gate_up(s, x16, table, counts, offsets, slot_token, h16, st, idx, dispatch_out);
     if (rc != ODSD_OK) return rc;
     rc = odsd_w4_down(s, h16, table, counts, offsets, y, st);
     if (rc != ODSD_OK) return rc;
@@ -808,7 +915,7 @@ int odsd_launch_experts(const odsd_moe_shape *s, const void *x16, const uint64_t
 int odsd_experts_dispatch_inside(const odsd_moe_shape *s) {
     if (experts_check(s) != ODSD_OK) return 0;
     const ExpertsPlan pl = experts_plan(s);
-    return pl.fused && odsd_fused_dispatch_supported(s->T * s->K);
+    return pl.fused ? odsd_fused_dispatch_supported(s->T * s->K) : stream_dispatch_supported(pl, s->T * s->K);
 }
 
 extern "C" int odsd_experts_w4(const odsd_moe_shape *s, const void *x_f16, const uint64_t *table,

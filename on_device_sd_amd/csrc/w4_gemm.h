@@ -29,6 +29,12 @@ struct GemmParams {
     int E;
     int n_wg;                // E * nchunks * KS (* PS)
     int wg_per_xcd;          // ceil(n_wg / 8)
+    // gate_up with the dispatch inside (idx given; counts / offsets / rowmap are then NOT inputs):
+    // every workgroup finds its expert's pairs in the id list itself, and the first workgroup of
+    // each expert leaves counts / offsets / perm for the down projection and the combine
+    const int32_t *idx;      // [P] expert id per (token, k) pair, or null
+    int32_t *out_counts, *out_offsets, *out_perm;
+    int K;
 };
 
 // Launch parameters of the one-launch expert kernel (experts_fused.hip)

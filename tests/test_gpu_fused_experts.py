@@ -133,3 +133,31 @@ def test_whole_block_dispatches_inside_the_expert_kernel(dev, layer, T):
     print(f"  vs oracle: max-abs {mx:.3e} mean-abs {mean:.3e}", flush=True)
     out2 = ops.moe_forward(x.to(dev), wg.to(dev), bank.table(), K, I, renorm=True)
     assert torch.equal(out2.out_f32, out.out_f32) and torch.equal(out2.perm, out.perm)
+
+
+def test_fused_experts_absent_and_substituted_experts(dev, layer):
+    """Table rows of the one-launch path: an expert without weights (row of zeros) contributes
+    nothing, as the reference skips experts without parameters (qwen3_runner.py:330-333); a row that
+    points at another expert's weights serves its own tokens with those weights (:322-329)."""
+    print("fused experts, absent and substituted experts", flush=True)
+    from on_device_sd_amd import ops
+    bank, experts = layer
+    T = 256
+    g = torch.Generator().manual_seed(77)
+    wg = (torch.randn(E, H, generator=g) * 0.02).to(torch.bfloat16)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    table = bank.table().clone()
+    absent, sub = (3, 64, 127), {5: 9, 100: 2}
+    for e in absent:
+        table[e] = 0
+    for e, src in sub.items():
+        table[e] = table[src]
+    out = ops.moe_forward(x.to(dev), wg.to(dev), table, K, I, renorm=True)
+    torch.cuda.synchronize()
+    idx, w = orc.route(orc.router_logits(x, wg), K, True)
+    assert np.array_equal(out.idx.cpu().numpy(), idx)
+    present = {e: ex for e, ex in experts.items() if e not in absent and e not in sub}
+    ref = orc.moe_forward(x, idx, w, present, substitution=sub)
+    mx, mean = check_output(out.out_f32, ref)
+    check_output_relative(out.out_f32, ref)
+    print(f"  vs oracle: max-abs {mx:.3e} mean-abs {mean:.3e}", flush=True)
