@@ -600,7 +600,9 @@ static ExpertsPlan experts_plan(const odsd_moe_shape *s) {
     // per expert, 128-row streaming passes up to ~130, the 256-row tile kernel beyond.
     p.tile = 0;
     if (s->T <= 16) p.MB = 1;
-    else if (s->T <= 32 || mean_rows <= 16) p.MB = 2;
+    else if (s->T <= 32) p.MB = 2;
+    else if (s->T <= 64) p.MB = 4;      // no expert can have more rows than a 64-row pass holds
+    else if (mean_rows <= 16) p.MB = 2;
     else if (mean_rows <= 52) p.MB = 4;
     else { p.MB = 8; p.tile = mean_rows > 136; }
     const long active = s->E < P ? s->E : P;       // upper bound of experts with rows
@@ -700,7 +702,7 @@ static void launch_gemm(GemmParams &gp, hipStream_t st) {
     gp.nchunks = (gp.NBLK + (WAVES / WK) * NB - 1) / ((WAVES / WK) * NB);
     gp.n_wg = gp.E * gp.nchunks * gp.KS;
     gp.wg_per_xcd = (gp.n_wg + 7) / 8;
-    if constexpr (MODE == 0 && MB == 2) {
+    if constexpr (MODE == 0 && !DIRECT && MB <= 4) {
         if (gp.idx) {
             ODSD_LAUNCH(ODSD_KERNEL_GATE_UP, (w4_gemm_kernel<NB, MB, MODE, DEPTH, NA, WK, DIRECT, OCC, WAVES, true>),
                         gp.wg_per_xcd * 8, 64 * WAVES, st, gp);
@@ -742,12 +744,13 @@ static int experts_args_ok(const odsd_moe_shape *s) {
 
 // gate_up + SiLU*mul: x_f16 [T,H] gathered by slot_token -> h_f16 [P,I] in slot order
 // the streaming gate_up kernels scan up to 4 ids per thread of their 256
-// (measured: with 32-row passes -- many experts, a dozen workgroups each -- the scan costs the
-// gate_up kernel nothing and saves the dispatch launch, 4 us of the Zipf-skewed T = 64 layer's 81;
-// with hundreds of workgroups per expert it costs gate_up more than the launch it saves: +7 us at
-// the Mixtral T = 160 shape, +6 us at T = 5, so those plans keep the dispatch kernel)
-static bool stream_dispatch_supported(const ExpertsPlan &pl, int P) {
-    return !pl.tile && pl.MB == 2 && P <= 4 * 256;
+// (measured: with a dozen workgroups per expert the scan costs the gate_up kernel nothing and saves
+// the dispatch launch, 4 us of the Zipf-skewed T = 64 layer's 81; with hundreds of workgroups per
+// expert it costs gate_up more than the launch it saves: +7 us at the Mixtral T = 160 shape, +6 us
+// at T = 5, so those plans keep the dispatch kernel)
+static bool stream_dispatch_supported(const ExpertsPlan &pl, const odsd_moe_shape *s) {
+    const int chunks = (2 * s->I / 16 + 4 * pl.NB - 1) / (4 * pl.NB);     // gate_up workgroups per expert
+    return !pl.tile && (pl.MB == 2 || pl.MB == 4) && chunks <= 32 && s->T * s->K <= 4 * 256;
 }
 
 // idx + dispatch_out: the dispatch arrays have not been filled; the kernel dispatches for itself
@@ -769,7 +772,7 @@ static int launch_gate_up(const odsd_moe_shape *s, const void *x_f16, const uint
     gu.KS = 1; gu.gper = gu.G; gu.PS = pl.PS_gu; gu.ldo = s->I; gu.P = s->T * s->K; gu.E = s->E;
     gu.K = s->K;
     if (dispatch_out) {
-        if (!stream_dispatch_supported(pl, gu.P)) return ODSD_ERR_UNSUPPORTED;
+        if (!stream_dispatch_supported(pl, s)) return ODSD_ERR_UNSUPPORTED;
         if (!idx || !dispatch_out->counts || !dispatch_out->offsets || !dispatch_out->perm) return ODSD_ERR_NULL;
         if (!odsd_aligned16(idx)) return ODSD_ERR_ALIGN;
         gu.idx = idx;
@@ -882,7 +885,7 @@ int odsd_launch_experts(const odsd_moe_shape *s, const void *x16, const uint64_t
     if (ws_bytes < pl.h_bytes + pl.y_bytes) return ODSD_ERR_WORKSPACE;
     void *h16 = ws;
     float *y = (float *)((char *)ws + pl.h_bytes);
-    if (dispatch_out && !(pl.fused ? odsd_fused_dispatch_supported(s->T * s->K) : stream_dispatch_supported(pl, s->T * s->K)))
+    if (dispatch_out && !(pl.fused ? odsd_fused_dispatch_supported(s->T * s->K) : stream_dispatch_supported(pl, s)))
         return ODSD_ERR_UNSUPPORTED;
     if (pl.fused) {
         if (!x16 || !table || !counts || !offsets || (!slot_token && !dispatch_out)) return ODSD_ERR_NULL;
@@ -915,7 +918,7 @@ int odsd_launch_experts(const odsd_moe_shape *s, const void *x16, const uint64_t
 int odsd_experts_dispatch_inside(const odsd_moe_shape *s) {
     if (experts_check(s) != ODSD_OK) return 0;
     const ExpertsPlan pl = experts_plan(s);
-    return pl.fused ? odsd_fused_dispatch_supported(s->T * s->K) : stream_dispatch_supported(pl, s->T * s->K);
+    return pl.fused ? odsd_fused_dispatch_supported(s->T * s->K) : stream_dispatch_supported(pl, s);
 }
 
 extern "C" int odsd_experts_w4(const odsd_moe_shape *s, const void *x_f16, const uint64_t *table,
