@@ -252,10 +252,6 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
                 wsz[slot][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_szd, (int)dsz_off, (tile + i * G_DN) * 64, 0);
             }
         };
-        // the ring's first loads depend on the table row only: they travel while the row map is
-        // read and the token rows are copied
-#pragma unroll
-        for (int d = 0; d < DEPTH; ++d) load_u(d, d);
         // rows past the expert's last one are clamped to the first row of the pass: the MFMA
         // columns they feed are never stored
         {
@@ -271,7 +267,12 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
                 }
             }
         }
-        ODSD_WAIT_VMCNT(0);                                   // the copies are the youngest requests
+        // The ring's first loads go out behind the copies and are not waited for: the group sums
+        // below run while they travel (issued in front of the copies they would have to land
+        // first -- the counter is in order -- and memory would idle during the sums: 1.3 us).
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) load_u(d, d);
+        ODSD_WAIT_VMCNT(4 * DEPTH);                           // the copies have landed; 4 loads per ring step are younger
         __builtin_amdgcn_s_barrier();
 
         // Sums of one (group, token block): the lane reads its four B fragments (token row r, columns
