@@ -6,8 +6,9 @@
 // step of 8 tokens and 8 query heads per KV head fills the 64 rows.  Each of the 4 wavefronts owns
 // 16 rows; the workgroup walks its keys 32 at a time:
 //   * the tile's K and V rows are fetched once per workgroup (two tiles ahead, into registers) and
-//     put into LDS one tile ahead: K as stored, V transposed; all wavefronts read their operands
-//     from there (double buffered, one barrier per tile);
+//     put into LDS one tile ahead, both as stored ([key][head_dim], 16- and 32-byte segments of a
+//     row XORed with the key against bank conflicts); all wavefronts read their operands from
+//     there (double buffered, one barrier per tile);
 //   * S^T = K Q^T on the matrix cores (v_mfma_f32_16x16x32, keys as the A operand, the
 //     wavefront's Q rows as the B operand held in registers), which leaves the scores of one
 //     query row in the 4 lanes that share lane % 16 -- the layout the P operand of the second
@@ -16,7 +17,9 @@
 //     value subtracted before exp2) follows its running maximum lazily, and the sum of the
 //     probabilities stays a per-lane partial sum until the end, so most tiles exchange nothing
 //     between lanes;
-//   * O += P V with V^T as the B operand.
+//   * O += P V with V^T as the B operand: a lane needs one head dimension of 8 keys, which
+//     ds_read_b64_tr_b16 delivers from the row-major tile (the 16 lanes of a group read 4 keys x
+//     16 dimensions and each gets one dimension's column of 4), so V is never transposed in memory.
 // A verify step has few (sequence, KV head) pairs and long key lists, so the keys of one sequence
 // are cut into `splits` slices handled by different workgroups; each leaves its reference point,
 // sum and unnormalised output, and a small second kernel merges the slices of a row (the usual
@@ -33,6 +36,7 @@
 #include <type_traits>
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float float2_t __attribute__((ext_vector_type(2)));
 
 struct AttnParams {
     const void *q;             // [n_tokens, H, HD]
@@ -49,7 +53,7 @@ struct AttnParams {
     // (contiguous, no block table); both null in paged mode
     const int32_t *cu_q, *cu_k;
     int splits;                // workgroups sharing one sequence's keys (blockIdx.z)
-    float *part;               // splits > 1: partial results [seq, kvh, row group][split][64][HD + 2]
+    float *part;               // splits > 1: partial results [seq, kvh, row group][split][64][HD + 4]
 };
 
 template <typename T> struct AttnT;
@@ -79,10 +83,6 @@ template <> struct AttnT<__bf16> {
     }
 };
 
-// position of key `key` (0..31) of a tile inside a row of the transposed V tile: the 8 keys a
-// lane group kq feeds to one product step (4 of each 16-key half) sit next to each other
-__device__ __forceinline__ int vt_pos(int key) { return 8 * ((key & 15) >> 2) + 4 * (key >> 4) + (key & 3); }
-
 // first query token of sequence seq: the sum of the query lengths before it, one wavefront-wide pass
 __device__ __forceinline__ int attn_first_token(const int32_t *q_lens, int seq) {
     int part = 0;
@@ -97,9 +97,11 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
     typedef typename AttnT<T>::V8 V8;
     constexpr int NJ = HD / 32;          // 32-dim steps of the score product
     constexpr int NDB = HD / 16;         // 16-dim column blocks of the output
-    constexpr int VT_LD = 40;            // halfs per row of the transposed V tile (32 keys + pad)
     constexpr int PIECES = 32 * (HD / 8) / 256;   // 16-byte pieces of a V tile per thread
-    __shared__ __attribute__((aligned(16))) uint16_t vt[2][HD * VT_LD];
+    // V tile as stored ([key][HD]); the 32-byte segment (16 dims) of a row is XORed with vswz(key):
+    // a transposing read touches 8 consecutive keys' segments of one column block per half wavefront
+    __shared__ __attribute__((aligned(16))) uint16_t vs[2][32 * HD];
+    auto vswz = [](int key) { return HD == 128 ? (key & 7) : ((key >> 1) & 3); };
     // K tile as stored ([key][HD]), 16-byte pieces of a row XORed with the key so that the 16 lanes
     // reading the same piece of 16 different keys hit different banks
     __shared__ __attribute__((aligned(16))) uint16_t kt[2][32 * HD];
@@ -155,7 +157,7 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
     // Software pipeline over the 32-key tiles, two tiles deep.  A tile's K and V rows are fetched
     // once per workgroup, 16 bytes per thread and piece (piece = tid + 256 u -> key = piece /
     // (HD / 8), dims 8 * (piece % (HD / 8)) ..), two tiles ahead into one of two register sets;
-    // one tile ahead they go to LDS -- K as stored, V transposed -- and every wavefront reads its
+    // one tile ahead they go to LDS, as stored, and every wavefront reads its
     // MFMA operands from there (K fetched per wavefront instead costs four times the L2 traffic
     // and was what bounded the kernel).  During tile `it`: the set that held tile `it` is refilled
     // with tile it + 2, the other set (tile it + 1) goes to the other LDS buffers, and the
@@ -227,11 +229,7 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
         for (int u = 0; u < PIECES; ++u) {
             const int piece = tid + 256 * u;
             const int key = piece / (HD / 8), ch = piece % (HD / 8);
-            const int pos = vt_pos(key) ^ (8 * (ch & 3));
-            const uint32_t w[4] = {vreg[S][u].x, vreg[S][u].y, vreg[S][u].z, vreg[S][u].w};
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-                vt[buf][(8 * ch + i) * VT_LD + pos] = (uint16_t)(w[i >> 1] >> (16 * (i & 1)));
+            *(uint4_t *)&vs[buf][key * HD + 16 * ((ch >> 1) ^ vswz(key)) + 8 * (ch & 1)] = vreg[S][u];
             *(uint4_t *)&kt[buf][key * HD + 8 * (ch ^ (key & (HD / 8 - 1)))] = kreg[S][u];
         }
     };
@@ -315,10 +313,20 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
             l_run += ((pe[0] + pe[1]) + (pe[2] + pe[3])) + ((pe[4] + pe[5]) + (pe[6] + pe[7]));
             const V8 pf = __builtin_bit_cast(V8, uint4_t{AttnT<T>::pack2(pe[0], pe[1]), AttnT<T>::pack2(pe[2], pe[3]),
                                                           AttnT<T>::pack2(pe[4], pe[5]), AttnT<T>::pack2(pe[6], pe[7])});
+            // B operand of column block db: dimension 16 db + c of keys 4 kq .. + 3 and 16 + 4 kq .. + 3
+            // (the keys of pf's 8 probabilities).  Lane c of a group addresses key 4 kq + c / 4,
+            // dimensions 16 db + 4 (c % 4) .. + 3; the read hands it column c of the group's 4 x 16 block.
+            const int key_a = 4 * kq + (c >> 2), key_b = key_a + 16;
+            const uint16_t *va = &vs[buf][key_a * HD + 4 * (c & 3)], *vb = &vs[buf][key_b * HD + 4 * (c & 3)];
+            const int swa = vswz(key_a), swb = vswz(key_b);
 #pragma unroll
             for (int db = 0; db < NDB; ++db) {
-                const int seg = kq ^ ((2 * db + (c >> 3)) & 3);
-                const V8 vf = __builtin_bit_cast(V8, *(const uint4_t *)&vt[buf][(16 * db + c) * VT_LD + 8 * seg]);
+                typedef short s4_t __attribute__((ext_vector_type(4)));
+                typedef __attribute__((address_space(3))) s4_t lds_s4;
+                const s4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4 *)(va + 16 * (db ^ swa)));
+                const s4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4 *)(vb + 16 * (db ^ swb)));
+                typedef short s8_t __attribute__((ext_vector_type(8)));
+                const V8 vf = __builtin_bit_cast(V8, s8_t{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w});
                 o[db] = AttnT<T>::mfma(pf, vf, o[db]);
             }
         }
@@ -366,16 +374,16 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
     l_run += __shfl_xor(l_run, 32, ODSD_WAVE);
     if (wave_active && p.splits > 1) {
         // partial result of this slice: rows of the workgroup's 64, [HD] unnormalised output, m, l
-        float *base = p.part + ((((size_t)blockIdx.x * gridDim.y + blockIdx.y) * p.splits + blockIdx.z) * 64) * (HD + 2);
+        float *base = p.part + ((((size_t)blockIdx.x * gridDim.y + blockIdx.y) * p.splits + blockIdx.z) * 64) * (HD + 4);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            float *rowp = base + (size_t)(wave * 16 + 4 * kq + i) * (HD + 2);
+            float *rowp = base + (size_t)(wave * 16 + 4 * kq + i) * (HD + 4);
 #pragma unroll
             for (int db = 0; db < NDB; ++db)
                 rowp[16 * db + c] = i == 0 ? o[db].x : i == 1 ? o[db].y : i == 2 ? o[db].z : o[db].w;
         }
         if (kq == 0) {
-            float *rowp = base + (size_t)(wave * 16 + c) * (HD + 2);
+            float *rowp = base + (size_t)(wave * 16 + c) * (HD + 4);
             rowp[HD] = m_run;
             rowp[HD + 1] = l_run;
         }
@@ -405,71 +413,93 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
 }
 
 // Merge of the key slices: out[row] = sum_s exp2(m_s - m) O_s / sum_s exp2(m_s - m) l_s, slices in
-// order. One workgroup per (sequence, KV head, row group, 256 / HD rows): a thread owns one output
-// element and walks the slices, neighbouring threads reading neighbouring floats.  (More rows per
-// workgroup, taken in turn, measured slower: each turn is one more exposed load latency.)
-template <typename T, int HD, int SB>
+// order. One workgroup per (sequence, KV head, row group, 256 VEC / HD rows): a thread owns VEC
+// neighbouring output elements of a row and walks the slices.  VEC = 4 (one 16-byte load per slice;
+// rows of the partial results are HD + 4 floats apart so that they stay 16-byte aligned) when there
+// are at most 4 slices: a quarter of the workgroups and of the exponentials; with more slices there
+// are few rows, and one element per thread keeps more of the chip busy.  (More rows per workgroup,
+// taken in turn, measured slower: each turn is one more exposed load latency.)
+template <typename T, int HD, int SB, int VEC>
 __global__ __launch_bounds__(256) void paged_attn_merge_kernel(const AttnParams p) {
-    constexpr int RPW = 256 / HD;                       // rows per workgroup
+    static_assert(VEC == 1 || VEC == 4, "one element or one 16-byte vector per thread");
+    constexpr int TPR = HD / VEC;                       // threads per row
+    constexpr int RPW = 256 / TPR;                      // rows per workgroup
     const int seq = blockIdx.x / p.KVH, kvh = blockIdx.x % p.KVH;
     const int Gq = p.H / p.KVH;
     const bool varlen = p.cu_k != nullptr;
     const int ql = varlen ? p.cu_q[seq + 1] - p.cu_q[seq] : (p.q_lens ? p.q_lens[seq] : 1);
     const int rows_total = ql * Gq;
     if ((varlen ? p.cu_k[seq + 1] - p.cu_k[seq] : p.context_lens[seq]) <= 0) return;
-    const int d = threadIdx.x % HD;
+    // the sequence's first token: a chain of its own (a wavefront-wide sum over the query lengths),
+    // started before the partial results are requested and by every lane of the wavefront
     int q0 = seq;
-    bool have_q0 = !p.q_lens || varlen;
     if (varlen) q0 = p.cu_q[seq];
-    {
-        const int r = (int)blockIdx.z * RPW + (int)threadIdx.x / HD;
-        const int row = (int)blockIdx.y * 64 + r;
-        if (row >= rows_total) return;                  // uniform per wavefront (HD >= 64)
-        const float *base = p.part + ((((size_t)blockIdx.x * gridDim.y + blockIdx.y) * p.splits) * 64 + r) * (HD + 2);
-        const size_t stride = (size_t)64 * (HD + 2);
-        // one pass, SB slices at a time (all their loads in flight together; SB = 4 when there are no
-        // more than 4 slices, so that none is fetched twice), rescaling the running
-        // sums whenever a batch raises the reference point
-        float m = -INFINITY, l = 0.0f, acc = 0.0f;
-        for (int s0 = 0; s0 < p.splits; s0 += SB) {
-            float ms[SB], ls[SB], os[SB];
+    else if (p.q_lens) q0 = attn_first_token(p.q_lens, seq);
+    const int d = VEC * ((int)threadIdx.x % TPR);
+    const int r = (int)blockIdx.z * RPW + (int)threadIdx.x / TPR;
+    const int row = (int)blockIdx.y * 64 + r;
+    if (row >= rows_total) return;
+    const float *base = p.part + ((((size_t)blockIdx.x * gridDim.y + blockIdx.y) * p.splits) * 64 + r) * (HD + 4);
+    const size_t stride = (size_t)64 * (HD + 4);
+    // one pass, SB slices at a time (all their loads in flight together; SB = 4 when there are no
+    // more than 4 slices, so that none is fetched twice), rescaling the running
+    // sums whenever a batch raises the reference point
+    float m = -INFINITY, l = 0.0f;
+    float acc[VEC];
 #pragma unroll
-            for (int u = 0; u < SB; ++u) {
-                // (every load unconditional, on a clamped slice: loads under a branch serialise)
-                const float *rp = base + (size_t)min(s0 + u, p.splits - 1) * stride;
-                ms[u] = rp[HD];
-                ls[u] = rp[HD + 1];
-                os[u] = rp[d];
+    for (int i = 0; i < VEC; ++i) acc[i] = 0.0f;
+    for (int s0 = 0; s0 < p.splits; s0 += SB) {
+        float ms[SB], ls[SB];
+        float os[SB][VEC];
+#pragma unroll
+        for (int u = 0; u < SB; ++u) {
+            // (every load unconditional, on a clamped slice: loads under a branch serialise)
+            const float *rp = base + (size_t)min(s0 + u, p.splits - 1) * stride;
+            const float2_t ml = *(const float2_t *)(rp + HD);
+            ms[u] = ml.x;
+            ls[u] = ml.y;
+            if constexpr (VEC == 4) {
+                const float4_t v = *(const float4_t *)(rp + d);
+                os[u][0] = v.x; os[u][1] = v.y; os[u][2] = v.z; os[u][3] = v.w;
+            } else {
+                os[u][0] = rp[d];
             }
-#pragma unroll
-            for (int u = 0; u < SB; ++u) {
-                if (s0 + u >= p.splits) {
-                    ms[u] = -INFINITY;
-                    ls[u] = os[u] = 0.0f;
-                }
-            }
-            float mb = m;
-#pragma unroll
-            for (int u = 0; u < SB; ++u) mb = fmaxf(mb, ms[u]);
-            const float ref = mb == -INFINITY ? 0.0f : mb;
-            const float keep = exp2f(m - ref);            // m = -inf -> 0
-            l *= keep;
-            acc *= keep;
-#pragma unroll
-            for (int u = 0; u < SB; ++u) {
-                const float f = exp2f(ms[u] - ref);
-                l += f * ls[u];
-                acc += f * os[u];
-            }
-            m = mb;
         }
-        if (!have_q0) {
-            q0 = attn_first_token(p.q_lens, seq);
-            have_q0 = true;
+#pragma unroll
+        for (int u = 0; u < SB; ++u) {
+            if (s0 + u >= p.splits) {
+                ms[u] = -INFINITY;
+                ls[u] = 0.0f;
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) os[u][i] = 0.0f;
+            }
         }
-        const float inv = l > 0.0f ? 1.0f / l : 0.0f;
-        const int tok = row / Gq, hq = row % Gq;
-        ((uint16_t *)p.out)[((size_t)(q0 + tok) * p.H + kvh * Gq + hq) * HD + d] = AttnT<T>::from_f32(acc * inv);
+        float mb = m;
+#pragma unroll
+        for (int u = 0; u < SB; ++u) mb = fmaxf(mb, ms[u]);
+        const float ref = mb == -INFINITY ? 0.0f : mb;
+        const float keep = exp2f(m - ref);            // m = -inf -> 0
+        l *= keep;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[i] *= keep;
+#pragma unroll
+        for (int u = 0; u < SB; ++u) {
+            const float f = exp2f(ms[u] - ref);
+            l += f * ls[u];
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[i] += f * os[u][i];
+        }
+        m = mb;
+    }
+    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+    const int tok = row / Gq, hq = row % Gq;
+    uint16_t *op = (uint16_t *)p.out + ((size_t)(q0 + tok) * p.H + kvh * Gq + hq) * HD + d;
+    if constexpr (VEC == 4) {
+        typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
+        *(u16x4 *)op = u16x4{AttnT<T>::from_f32(acc[0] * inv), AttnT<T>::from_f32(acc[1] * inv),
+                             AttnT<T>::from_f32(acc[2] * inv), AttnT<T>::from_f32(acc[3] * inv)};
+    } else {
+        op[0] = AttnT<T>::from_f32(acc[0] * inv);
     }
 }
 
@@ -497,7 +527,7 @@ extern "C" size_t odsd_paged_attention_workspace_bytes(int32_t n_seqs, int32_t m
     const int rg = (int)((rows + 63) / 64);
     const int splits = attn_splits(n_seqs, num_kv_heads, rg, max_blocks, block_size);
     if (splits == 1) return 256;
-    return odsd_round_up((size_t)n_seqs * num_kv_heads * rg * splits * 64 * (head_dim + 2) * sizeof(float), 256);
+    return odsd_round_up((size_t)n_seqs * num_kv_heads * rg * splits * 64 * (head_dim + 4) * sizeof(float), 256);
 }
 
 extern "C" int odsd_paged_attention(const void *q, const void *k_cache, const void *v_cache,
@@ -535,14 +565,15 @@ extern "C" int odsd_paged_attention(const void *q, const void *k_cache, const vo
         p.part = (float *)workspace;
     }
     const dim3 grid((unsigned)(n_seqs * num_kv_heads), (unsigned)rg, (unsigned)p.splits);
-    const dim3 mgrid((unsigned)(n_seqs * num_kv_heads), (unsigned)rg, (unsigned)(64 / (256 / head_dim)));
+    const int mvec = p.splits > 4 ? 1 : 4;
+    const dim3 mgrid((unsigned)(n_seqs * num_kv_heads), (unsigned)rg, (unsigned)(64 / (256 * mvec / head_dim)));
     hipStream_t st = (hipStream_t)stream;
 #define ATTN_GO(T, HDV)                                                              \
     do {                                                                             \
         if (block_size % 32 == 0) paged_attn_kernel<T, HDV, true><<<grid, 256, 0, st>>>(p);  \
         else paged_attn_kernel<T, HDV, false><<<grid, 256, 0, st>>>(p);              \
-        if (p.splits > 4) paged_attn_merge_kernel<T, HDV, 8><<<mgrid, 256, 0, st>>>(p);      \
-        else if (p.splits > 1) paged_attn_merge_kernel<T, HDV, 4><<<mgrid, 256, 0, st>>>(p); \
+        if (p.splits > 4) paged_attn_merge_kernel<T, HDV, 8, 1><<<mgrid, 256, 0, st>>>(p);      \
+        else if (p.splits > 1) paged_attn_merge_kernel<T, HDV, 4, 4><<<mgrid, 256, 0, st>>>(p); \
     } while (0)
     if (dtype == ODSD_DT_F16) {
         if (head_dim == 128) ATTN_GO(half_t, 128);
@@ -597,13 +628,14 @@ extern "C" int odsd_varlen_attention(const void *q, const void *k, const void *v
         p.part = (float *)workspace;
     }
     const dim3 grid((unsigned)(n_seqs * num_kv_heads), (unsigned)rg, (unsigned)p.splits);
-    const dim3 mgrid((unsigned)(n_seqs * num_kv_heads), (unsigned)rg, (unsigned)(64 / (256 / head_dim)));
+    const int mvec = p.splits > 4 ? 1 : 4;
+    const dim3 mgrid((unsigned)(n_seqs * num_kv_heads), (unsigned)rg, (unsigned)(64 / (256 * mvec / head_dim)));
     hipStream_t st = (hipStream_t)stream;
 #define ATTN_GO(T, HDV)                                                              \
     do {                                                                             \
         paged_attn_kernel<T, HDV, true><<<grid, 256, 0, st>>>(p);                    \
-        if (p.splits > 4) paged_attn_merge_kernel<T, HDV, 8><<<mgrid, 256, 0, st>>>(p);      \
-        else if (p.splits > 1) paged_attn_merge_kernel<T, HDV, 4><<<mgrid, 256, 0, st>>>(p); \
+        if (p.splits > 4) paged_attn_merge_kernel<T, HDV, 8, 1><<<mgrid, 256, 0, st>>>(p);      \
+        else if (p.splits > 1) paged_attn_merge_kernel<T, HDV, 4, 4><<<mgrid, 256, 0, st>>>(p); \
     } while (0)
     if (dtype == ODSD_DT_F16) {
         if (head_dim == 128) ATTN_GO(half_t, 128);
