@@ -104,13 +104,16 @@ int odsd_launch_dispatch(const odsd_moe_shape *s, const int32_t *idx, int32_t *c
     if (!idx || !counts || !offsets || !perm || !inv || !slot_token) return ODSD_ERR_NULL;
     if (s->T == 0) return ODSD_OK;
     const int P = s->T * s->K;
-    const int threads = P <= 4096 ? 256 : 1024;
+    // wavefronts per workgroup: enough that a wavefront keeps at most 4 x 64 ids where the pair list
+    // allows it (the register-resident forms unroll ITERS loads and 4 ITERS ballots per wavefront)
+    const int threads = P <= 1024 ? 256 : (P <= 2048 ? 512 : 1024);
     const int nwaves = threads / 64;
     const int iters = (((P + nwaves - 1) / nwaves + 63) & ~63) / 64;   // 64-pair chunks per wavefront
 #define DISPATCH_GO(IT)                                                                            \
     ODSD_LAUNCH(ODSD_KERNEL_DISPATCH, dispatch_kernel<IT>, s->E, threads, st, idx, P, s->K, s->E, counts, \
                 offsets, perm, inv, slot_token)
     if (iters <= 2) DISPATCH_GO(2);
+    else if (iters <= 4) DISPATCH_GO(4);
     else if (iters <= 8) DISPATCH_GO(8);
     else if (iters <= 32) DISPATCH_GO(32);
     else DISPATCH_GO(0);

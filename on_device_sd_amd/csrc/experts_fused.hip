@@ -76,12 +76,13 @@ typedef float float2_t __attribute__((ext_vector_type(2)));
 // WAVES wavefronts per workgroup
 // G_UP  H / 128, G_DN  I / 128: groups of the two reductions (compile time: every tile offset of
 //       a wavefront's stream is a constant)
-// DISP  the workgroup dispatches for itself: it scans the [P] expert ids (P <= 4 * 64 * WAVES, one
-//       vector of 4 per thread), counts the pairs of its expert and of lower experts (ballot /
+// DISP  0, or the number of 4-id vectors per thread (1 or 2) with which the workgroup dispatches
+//       for itself: it scans the [P] expert ids (P <= 4 * DISP * 64 * WAVES, consecutive ids per
+//       thread), counts the pairs of its expert and of lower experts (ballot /
 //       popcount, the order of the pair list is kept: stable), keeps its expert's token rows in LDS
 //       and, as slice 0, writes counts[e], offsets[e] and the slots of its pairs -- what the
 //       separate dispatch kernel and two dependent loads per workgroup did before
-template <int MB, int GS, int WAVES, int G_UP, int G_DN, bool DISP>
+template <int MB, int GS, int WAVES, int G_UP, int G_DN, int DISP>
 __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(const FusedParams p) {
     static_assert(WAVES % 4 == 0 && (8 * GS) % WAVES == 0, "whole gate/up block pairs per wavefront");
     static_assert(G_UP * MB <= ODSD_FUSED_X_BLOCKS, "token rows of a pass must fit the LDS area");
@@ -108,29 +109,40 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
     const uint64_t *trow = p.table + (size_t)e * ODSD_TABLE_COLS;
     const uint64_t t_gu_q = trow[0], t_gu_sz = trow[1], t_dn_q = trow[2], t_dn_sz = trow[3];
     int M_e, base;
-    int rk[4] = {-1, -1, -1, -1};                // DISP: rank of this thread's pairs inside the expert, or -1
+    constexpr int NID = DISP ? 4 * DISP : 1;     // ids per thread
+    int rk[NID];                                 // DISP: rank of this thread's pairs inside the expert, or -1
+#pragma unroll
+    for (int j = 0; j < NID; ++j) rk[j] = -1;
     int pair0 = 0;
     if (DISP) {
         const int tid_ = threadIdx.x, lane_ = tid_ & 63, wave_ = tid_ >> 6;
-        pair0 = 4 * tid_;
-        int id[4] = {-1, -1, -1, -1};
-        if (pair0 < p.P) {                       // P is a multiple of 4
-            const uint4_t v = *(const uint4_t *)(p.idx + pair0);
-            id[0] = (int)v.x; id[1] = (int)v.y; id[2] = (int)v.z; id[3] = (int)v.w;
+        pair0 = NID * tid_;
+        int id[NID];
+#pragma unroll
+        for (int v = 0; v < NID / 4; ++v) {
+            uint4_t w = {~0u, ~0u, ~0u, ~0u};
+            if (pair0 + 4 * v < p.P) w = *(const uint4_t *)(p.idx + pair0 + 4 * v);   // P is a multiple of 4
+            id[4 * v] = (int)w.x; id[4 * v + 1] = (int)w.y; id[4 * v + 2] = (int)w.z; id[4 * v + 3] = (int)w.w;
         }
         int cm = 0, cl = 0;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < NID; ++j) {
             cm += id[j] == e;
             cl += (uint32_t)id[j] < (uint32_t)e; // ids outside [0, E) belong to nobody
         }
-        // counts of at most 4 per lane: three ballots give the prefix over the lower lanes and the total
-        const uint64_t m0b = __ballot(cm & 1), m1b = __ballot(cm & 2), m2b = __ballot(cm & 4);
-        const uint64_t l0b = __ballot(cl & 1), l1b = __ballot(cl & 2), l2b = __ballot(cl & 4);
-        const int pre = mask_rank(m0b) + 2 * mask_rank(m1b) + 4 * mask_rank(m2b);
+        // counts of at most NID per lane: one ballot per bit gives the prefix over the lower lanes and the total
+        constexpr int NBITS = DISP == 1 ? 3 : 4;
+        int pre = 0, tot_eq = 0, tot_lt = 0;
+#pragma unroll
+        for (int b = 0; b < NBITS; ++b) {
+            const uint64_t mb = __ballot(cm & (1 << b)), lb = __ballot(cl & (1 << b));
+            pre += mask_rank(mb) << b;
+            tot_eq += __popcll(mb) << b;
+            tot_lt += __popcll(lb) << b;
+        }
         if (lane_ == 0) {
-            wsum[0][wave_] = __popcll(m0b) + 2 * __popcll(m1b) + 4 * __popcll(m2b);
-            wsum[1][wave_] = __popcll(l0b) + 2 * __popcll(l1b) + 4 * __popcll(l2b);
+            wsum[0][wave_] = tot_eq;
+            wsum[1][wave_] = tot_lt;
         }
         __syncthreads();
         int before = 0, tot_m = 0, tot_l = 0;
@@ -145,7 +157,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
         base = tot_l;
         int rank = before + pre;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < NID; ++j) {
             if (id[j] == e) rk[j] = rank++;
         }
         if (s == 0) {
@@ -155,7 +167,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
                 if (e == p.E - 1) p.out_offsets[p.E] = base + M_e;
             }
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < NID; ++j) {
                 // (the ids come from this library's router, so every pair belongs to some expert's workgroup)
                 if (rk[j] >= 0) p.out_perm[pair0 + j] = base + rk[j];
             }
@@ -221,7 +233,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
         if (DISP) {
             // tokens of this pass's rows (readers of the previous pass's list passed several barriers ago)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < NID; ++j) {
                 const int rel = rk[j] - m0;
                 if (rk[j] >= 0 && rel >= 0 && rel < 16 * MB) rows_lds[rel] = (pair0 + j) / p.K;
             }
@@ -440,14 +452,16 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
 // Shapes the fused kernel is built for; the caller has checked them with odsd_fused_supported().
 void odsd_launch_experts_fused(FusedParams &fp, int E, hipStream_t st) {
     // (MB = 2: up to 32 rows per pass; experts with at most 16 rows skip the second token block)
-    if (fp.idx)
-        ODSD_LAUNCH(ODSD_KERNEL_EXPERTS, (w4_expert_fused_kernel<2, 3, 8, 16, 6, true>), E * fp.S, 512, st, fp);
+    if (fp.idx && fp.P <= 4 * 512)
+        ODSD_LAUNCH(ODSD_KERNEL_EXPERTS, (w4_expert_fused_kernel<2, 3, 8, 16, 6, 1>), E * fp.S, 512, st, fp);
+    else if (fp.idx)
+        ODSD_LAUNCH(ODSD_KERNEL_EXPERTS, (w4_expert_fused_kernel<2, 3, 8, 16, 6, 2>), E * fp.S, 512, st, fp);
     else
-        ODSD_LAUNCH(ODSD_KERNEL_EXPERTS, (w4_expert_fused_kernel<2, 3, 8, 16, 6, false>), E * fp.S, 512, st, fp);
+        ODSD_LAUNCH(ODSD_KERNEL_EXPERTS, (w4_expert_fused_kernel<2, 3, 8, 16, 6, 0>), E * fp.S, 512, st, fp);
 }
 
-// the in-kernel dispatch holds the whole id list in one vector of 4 ids per thread
-int odsd_fused_dispatch_supported(int P) { return P % 4 == 0 && P <= 4 * 512; }
+// the in-kernel dispatch holds the whole id list in one or two vectors of 4 ids per thread
+int odsd_fused_dispatch_supported(int P) { return P % 4 == 0 && P <= 8 * 512; }
 
 // H = 2048 (4 sub-passes of 8 wavefronts x 4 blocks), slices of 384 features, token rows of one
 // pass within the 128 KB row area

@@ -109,7 +109,7 @@ def test_fused_experts_vs_stages_and_oracle(dev, layer, T, forced):
     assert torch.equal(out32b, out32)
 
 
-@pytest.mark.parametrize("T", [256, 136])
+@pytest.mark.parametrize("T", [256, 136, 320, 300])
 def test_whole_block_dispatches_inside_the_expert_kernel(dev, layer, T):
     """odsd_moe_forward at this shape launches no dispatch kernel: the expert kernel's workgroups
     scan the expert ids themselves.  Indices, counts, offsets and the permutation must still be
