@@ -221,8 +221,7 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
             }
         }
     };
-    // V^T tile in LDS: row = dim, 32 key positions (+ pad); the 8-position segment index is XORed
-    // with (dim / 8) & 3 so that the 16 lanes writing one key's 16 dim chunks spread over the banks
+    // a tile's K and V rows into the LDS buffers `buf`, 16 bytes per thread and piece, as stored
     auto store_kv = [&](auto set, int buf) {
         constexpr int S = decltype(set)::value;
 #pragma unroll
