@@ -46,8 +46,9 @@
 extern "C" {
 #endif
 
-/* 110: events / static forms of the whole block, KV store, paged and packed attention added (100: the MoE block) */
-#define ODSD_VERSION 111
+/* 110: events / static forms of the whole block, KV store, paged and packed attention added (100: the MoE block)
+ * 112: odsd_moe_shape.max_rows (was reserved, 0 keeps the old meaning), odsd_experts_one_launch */
+#define ODSD_VERSION 112
 
 typedef enum odsd_status {
     ODSD_OK = 0,
@@ -72,7 +73,12 @@ typedef struct odsd_moe_shape {
                            1: those weights divided by their sum (== softmax over the K
                               selected logits, the demo engine's top-k -> softmax)        */
     int32_t act_dtype;  /* dtype of x, gate weight, residual and out_act                 */
-    int32_t reserved;
+    int32_t max_rows;   /* 0: not known.  > 0: the caller states that no expert has more (token, k)
+                           pairs than this in the call -- it has read the per-expert counts, as
+                           the reference engine does between route_experts and forward_moe
+                           (qwen3_runner.py:110-112).  The experts calls then stay away from a
+                           plan that would stream an expert's weights a second time for a few
+                           rows.  A wrong value costs time, never correctness.              */
 } odsd_moe_shape;
 
 /* Per-expert weight table: E rows of 4 device addresses (as uint64):
@@ -178,6 +184,13 @@ int     odsd_w4_gate_up_silu(const odsd_moe_shape *s, const void *x_f16, const u
                              const int32_t *counts, const int32_t *offsets,
                              const int32_t *slot_token, void *h_f16, void *stream);
 int32_t odsd_w4_down_splits(const odsd_moe_shape *s);
+/* 1 if odsd_experts_w4 / odsd_moe_forward run gate_up, SiLU*mul and down of this shape in one
+ * launch (one workgroup per expert slice, token rows resident in LDS, at most
+ * ODSD_ONE_LAUNCH_ROWS rows of an expert per pass over its weights), 0 if they run the two
+ * launches of the stage calls, negative status for a bad shape.  (A planning query: no
+ * counterpart in the reference, whose per-expert loop has no such choice.) */
+#define ODSD_ONE_LAUNCH_ROWS 32
+int32_t odsd_experts_one_launch(const odsd_moe_shape *s);
 int     odsd_w4_down(const odsd_moe_shape *s, const void *h_f16, const uint64_t *table,
                      const int32_t *counts, const int32_t *offsets, void *y, void *stream);
 int     odsd_combine(const odsd_moe_shape *s, const void *y, const int32_t *idx, const float *w,

@@ -23,7 +23,7 @@ class MoeShape(C.Structure):
     """Mirror of ``odsd_moe_shape``."""
     _fields_ = [("T", C.c_int32), ("H", C.c_int32), ("E", C.c_int32), ("K", C.c_int32),
                 ("I", C.c_int32), ("renorm", C.c_int32), ("act_dtype", C.c_int32),
-                ("reserved", C.c_int32)]
+                ("max_rows", C.c_int32)]
 
 
 _P = C.c_void_p
@@ -49,6 +49,7 @@ SIGNATURES = {
     "odsd_experts_w4": (C.c_int, [_SP, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, C.c_size_t, _P]),
     "odsd_w4_gate_up_silu": (C.c_int, [_SP, _P, _P, _P, _P, _P, _P, _P]),
     "odsd_w4_down_splits": (C.c_int32, [_SP]),
+    "odsd_experts_one_launch": (C.c_int32, [_SP]),
     "odsd_w4_down": (C.c_int, [_SP, _P, _P, _P, _P, _P, _P]),
     "odsd_combine": (C.c_int, [_SP, _P, _P, _P, _P, _P, _P, _P, _P, _P]),
     "odsd_moe_workspace_bytes": (C.c_size_t, [_SP]),

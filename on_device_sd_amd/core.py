@@ -47,6 +47,9 @@ class RoutingResult:
     # the routed tensor itself: while the routing result lives, its storage cannot be handed to
     # another tensor, so the address in x_tag keeps meaning "that tensor"
     x_src: Optional[torch.Tensor] = field(default=None, repr=False, compare=False)
+    # the largest per-expert pair count, read on the host together with the activated set
+    # (0: not known); forward_moe hands it to the library with the dispatch arrays it belongs to
+    max_rows: int = field(default=0, repr=False, compare=False)
 
     @property
     def top_k(self) -> int:

@@ -661,9 +661,13 @@ static ExpertsPlan experts_plan(const odsd_moe_shape *s) {
     // need a second pass over their weights): one workgroup per
     // (expert, slice of the intermediate dimension), E * S workgroups for 256 CUs.  The stage entry
     // points keep the two-launch plan above; only the whole-block calls take this path.
+    // An expert with more rows than a pass holds streams its slice a second time while the other
+    // CUs have nothing left to do (110 against 84 us for the layer with one expert at 33 rows; the
+    // two-launch plan stays at 85): a caller that knows the largest count says so in max_rows, and
+    // the plan then takes the one-launch kernel only when one pass covers every expert.
     p.fused = 0;
     p.S = 1;
-    if (s->T > 16 && mean_rows >= 8 && mean_rows <= 20) {
+    if (s->T > 16 && mean_rows >= 8 && mean_rows <= 20 && (s->max_rows <= 0 || s->max_rows <= ODSD_ONE_LAUNCH_ROWS)) {
         int S = 256 / s->E;
         if (S >= 1 && S <= 2 && s->E * S >= 192 && odsd_fused_supported(s->H, s->I, S)) {
             p.fused = 1;
@@ -792,6 +796,12 @@ extern "C" int odsd_w4_gate_up_silu(const odsd_moe_shape *s, const void *x_f16, 
 extern "C" int32_t odsd_w4_down_splits(const odsd_moe_shape *s) {
     if (experts_check(s) != ODSD_OK) return 0;
     return experts_plan(s).KS;
+}
+
+extern "C" int32_t odsd_experts_one_launch(const odsd_moe_shape *s) {
+    const int rc = experts_check(s);
+    if (rc != ODSD_OK) return -rc;
+    return experts_plan(s).fused;
 }
 
 // down: h_f16 [P,I] -> y [KS][P][H] fp32 partial sums over KS slices of I

@@ -452,6 +452,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
 // Shapes the fused kernel is built for; the caller has checked them with odsd_fused_supported().
 void odsd_launch_experts_fused(FusedParams &fp, int E, hipStream_t st) {
     // (MB = 2: up to 32 rows per pass; experts with at most 16 rows skip the second token block)
+    static_assert(ODSD_ONE_LAUNCH_ROWS == 16 * 2, "rows of one pass as the header states them");
     if (fp.idx && fp.P <= 4 * 512)
         ODSD_LAUNCH(ODSD_KERNEL_EXPERTS, (w4_expert_fused_kernel<2, 3, 8, 16, 6, 1>), E * fp.S, 512, st, fp);
     else if (fp.idx)

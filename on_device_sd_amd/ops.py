@@ -38,8 +38,10 @@ def _require_cuda(*tensors: torch.Tensor) -> None:
                                "(there is no CPU fallback)")
 
 
-def make_shape(T: int, H: int, E: int, K: int, I: int, renorm: bool, dtype: torch.dtype) -> MoeShape:
-    return MoeShape(T, H, E, K, I, 1 if renorm else 0, _dtype_code(dtype), 0)
+def make_shape(T: int, H: int, E: int, K: int, I: int, renorm: bool, dtype: torch.dtype,
+               max_rows: int = 0) -> MoeShape:
+    """``max_rows``: the largest per-expert pair count if the caller knows it (0: unknown)."""
+    return MoeShape(T, H, E, K, I, 1 if renorm else 0, _dtype_code(dtype), max(0, int(max_rows)))
 
 
 def _workspace(nbytes: int, device) -> torch.Tensor:
@@ -259,9 +261,11 @@ def route_dispatch(x: torch.Tensor, gate_weight: torch.Tensor, top_k: int, renor
 def experts_w4(x_f16: torch.Tensor, table: torch.Tensor, idx: torch.Tensor, w: torch.Tensor,
                disp: Dispatch, inter: int, act_dtype: torch.dtype,
                residual: Optional[torch.Tensor] = None, want_f32: bool = True,
-               want_act: bool = False):
+               want_act: bool = False, max_rows: int = 0):
     """Grouped W4 SwiGLU over the dispatched pairs and the weighted combine.
-    Returns (out_f32 or None, out_act or None), both [T, H]."""
+    Returns (out_f32 or None, out_act or None), both [T, H].  ``max_rows``: the largest
+    per-expert count if the caller has read the counts (0: unknown); with it the library avoids a
+    plan that would stream an expert's weights twice for a few rows."""
     _require_cuda(x_f16, table, idx, w)
     lib = _lib.load()
     T, H = x_f16.shape
@@ -269,7 +273,7 @@ def experts_w4(x_f16: torch.Tensor, table: torch.Tensor, idx: torch.Tensor, w: t
     K = idx.shape[1]
     if idx.dtype != torch.int32:
         idx = idx.to(torch.int32)
-    shape = make_shape(T, H, E, K, inter, False, act_dtype)
+    shape = make_shape(T, H, E, K, inter, False, act_dtype, max_rows)
     dev = x_f16.device
     out32 = torch.empty(T, H, dtype=torch.float32, device=dev) if want_f32 else None
     outa = torch.empty(T, H, dtype=act_dtype, device=dev) if want_act else None

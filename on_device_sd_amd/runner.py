@@ -77,7 +77,8 @@ class W4MoERunner:
         activated = set(map(ids.__getitem__, self._counts_np.nonzero()[0].tolist()))
         return RoutingResult(layer_idx=layer_idx, topk_indices=idx64, topk_scores=w,
                              activated_expert_ids=activated, dispatch=disp, x_f16=x16,
-                             x_tag=_tensor_tag(flat), x_src=hidden_states)
+                             x_tag=_tensor_tag(flat), x_src=hidden_states,
+                             max_rows=int(self._counts_np.max()) if self._counts_np.size else 0)
 
     def forward_moe(self, layer_idx: int, attn_output: AttentionOutput,
                     expert_placement: ExpertPlacement) -> torch.Tensor:
@@ -169,7 +170,8 @@ class W4MoERunner:
             else ops.to_f16(flat)
         _, out = ops.experts_w4(x16, table, idx, scores, disp,
                                 self.config.moe_intermediate_size, flat.dtype, residual=res,
-                                want_f32=False, want_act=True)
+                                want_f32=False, want_act=True,
+                                max_rows=routing.max_rows if routing.dispatch is not None else 0)
         return out.view(shape)
 
 

@@ -27,10 +27,27 @@ def test_every_declared_symbol_is_exported_and_bound():
 
 def test_version_and_status_strings():
     lib = _lib.load()
-    assert lib.odsd_version() == 111
+    assert lib.odsd_version() == 112
     assert lib.odsd_status_string(0) == b"ok"
     for code in range(1, 9):
         assert len(lib.odsd_status_string(code)) > 3
+
+
+def test_one_launch_plan_follows_shape_and_max_rows():
+    """The whole-block experts calls take the one-launch kernel at the Qwen3-30B expert shape with
+    8 to 20 rows per expert on average, unless the caller says that some expert has more rows than
+    one pass of that kernel holds (the counts the reference engine reads on the host between
+    route_experts and forward_moe, qwen3_runner.py:110-112)."""
+    lib = _lib.load()
+    q = lambda T, mr: lib.odsd_experts_one_launch(C.byref(_lib.MoeShape(T, 2048, 128, 8, 768, 1, _lib.DT_BF16, mr)))
+    assert q(256, 0) == 1 and q(128, 0) == 1 and q(320, 0) == 1
+    assert q(256, 32) == 1 and q(256, 33) == 0 and q(256, 70) == 0
+    assert q(64, 0) == 0 and q(384, 0) == 0 and q(4096, 0) == 0          # too few / too many rows per expert
+    assert lib.odsd_experts_one_launch(C.byref(_lib.MoeShape(160, 4096, 8, 2, 14336, 0, _lib.DT_BF16, 0))) == 0
+    assert lib.odsd_experts_one_launch(C.byref(_lib.MoeShape(160, 4000, 8, 2, 14336, 0, _lib.DT_BF16, 0))) == -2
+    # the workspace answer does not depend on the statement (one buffer serves either plan)
+    ws = lambda mr: lib.odsd_experts_workspace_bytes(C.byref(_lib.MoeShape(256, 2048, 128, 8, 768, 1, _lib.DT_BF16, mr)))
+    assert ws(0) == ws(40) > 0
 
 
 def test_argument_checks_need_no_gpu():

@@ -161,3 +161,46 @@ def test_fused_experts_absent_and_substituted_experts(dev, layer):
     mx, mean = check_output(out.out_f32, ref)
     check_output_relative(out.out_f32, ref)
     print(f"  vs oracle: max-abs {mx:.3e} mean-abs {mean:.3e}", flush=True)
+
+
+def test_max_rows_statement_takes_the_two_launch_plan(dev, layer):
+    """An expert with more rows than one pass of the one-launch kernel holds makes that kernel
+    stream the expert's weights twice; a caller that has read the counts (route_experts does, as
+    qwen3_runner.py:110-112) passes the largest one along, and the call runs the two-launch plan
+    instead.  Both answers are the oracle's within tolerance, and the runner's two-call path
+    carries the count by itself."""
+    print("fused experts, max_rows statement", flush=True)
+    import ctypes as C
+    import on_device_sd_amd as odsd
+    from on_device_sd_amd import _lib, ops
+    bank, experts = layer
+    T = 256
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    idx_np = _routing(T, {5: 40, 77: 3}, seed=9)
+    w_np = np.random.default_rng(3).random((T, K), dtype=np.float32)
+    w_np /= w_np.sum(axis=1, keepdims=True)
+    idx = torch.from_numpy(idx_np).to(torch.int32).to(dev)
+    w = torch.from_numpy(w_np).to(dev)
+    x16 = ops.to_f16(x.to(dev))
+    disp = ops.dispatch(idx, E)
+    lib = _lib.load()
+    assert lib.odsd_experts_one_launch(C.byref(ops.make_shape(T, H, E, K, I, False, torch.bfloat16))) == 1
+    assert lib.odsd_experts_one_launch(C.byref(ops.make_shape(T, H, E, K, I, False, torch.bfloat16, 40))) == 0
+    one, _ = ops.experts_w4(x16, bank.table(), idx, w, disp, I, torch.bfloat16, want_f32=True)
+    two, _ = ops.experts_w4(x16, bank.table(), idx, w, disp, I, torch.bfloat16, want_f32=True, max_rows=40)
+    torch.cuda.synchronize()
+    ref = orc.moe_forward(x, idx_np, w_np, experts)
+    for out in (one, two):
+        check_output(out, ref)
+        check_output_relative(out, ref)
+    d = (one - two).abs().max().item()
+    print(f"  one-launch vs two-launch plan: max-abs {d:.3e}", flush=True)
+    assert d <= 2e-3 * ref.abs().max().item()
+    # the engine path: route_experts reads the counts and notes the largest
+    cfg = odsd.MoEConfig(hidden_size=H, num_hidden_layers=1, num_experts=E, num_experts_per_token=K,
+                         moe_intermediate_size=I, norm_topk_prob=True)
+    wg = (torch.randn(E, H, generator=g) * 0.02).to(torch.bfloat16)
+    runner = odsd.W4MoERunner(cfg, [wg.to(dev)], [bank])
+    routing = runner.route_experts(0, x.to(dev))
+    assert routing.max_rows == int(routing.dispatch.counts.max().item()) > 0
