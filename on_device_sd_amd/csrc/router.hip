@@ -331,16 +331,19 @@ struct RouterPlan {
     size_t partial_bytes;
 };
 
-static RouterPlan router_plan(const odsd_moe_shape *s) {
+static RouterPlan router_plan(const odsd_moe_shape *s, bool normed) {
     RouterPlan p;
     const int ET = (s->E + 15) / 16;
     p.TT = (s->T + 15) / 16;
     // Expert tiles per wavefront: more of them re-use a token chunk more often, fewer give more and
     // shorter wavefront units.  With few 16 x 16 output tiles the kernel is a latency chain and short
     // units win (E = 128: 4.6 against 6.9 us at T = 128, 6.5 against 7.1 at 256, 8.4 against 10.6 at
-    // 320); from ~512 tiles on the re-use wins (T = 4096, H = 4096: 94 against 117 us).
+    // 320); from ~512 tiles on the re-use wins (T = 4096, H = 4096: 94 against 117 us).  With the
+    // RMSNorm folded in, every expert group also repeats the normalisation of its token chunk (two
+    // fp64 conversions per element): two tiles per wavefront are then the least (T = 256 in the
+    // 48-layer stack: 8.2 us against 9.3 with one, 8.3 with four).
     const long tiles = (long)p.TT * ET;
-    const int ne = tiles <= 192 ? 1 : (tiles <= 512 ? 2 : 4);
+    const int ne = tiles <= 192 ? (normed ? 2 : 1) : (tiles <= 512 ? 2 : 4);
     p.NE = ET >= ne ? ne : (ET >= 2 ? 2 : 1);
     p.EG = (ET + p.NE - 1) / p.NE;
     // split K until there are ~2048 wavefront units or the slices get down to 64 columns
@@ -366,7 +369,9 @@ static int router_check(const odsd_moe_shape *s) {
 
 extern "C" size_t odsd_router_workspace_bytes(const odsd_moe_shape *s) {
     if (router_check(s) != ODSD_OK) return 0;
-    return router_plan(s).partial_bytes;
+    // (the split of K, and with it the partial sums, depends on whether the RMSNorm is folded in)
+    const size_t a = router_plan(s, false).partial_bytes, b = router_plan(s, true).partial_bytes;
+    return a > b ? a : b;
 }
 
 template <typename XT, int NE>
@@ -398,7 +403,7 @@ int odsd_launch_router(const odsd_moe_shape *s, const void *x, const void *gate_
     if (!odsd_aligned16(x) || !odsd_aligned16(gate_w) || !odsd_aligned16(ws) ||
         (x16 && !odsd_aligned16(x16)))
         return ODSD_ERR_ALIGN;
-    const RouterPlan p = router_plan(s);
+    const RouterPlan p = router_plan(s, norm_ss != nullptr);
     if (ws_bytes < p.partial_bytes) return ODSD_ERR_WORKSPACE;
     double *partial = (double *)ws;
     const bool bf = s->act_dtype == ODSD_DT_BF16;
