@@ -340,6 +340,11 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
             ODSD_FENCE();
             refill();                                         // the slot is free again
             ODSD_FENCE();
+            // The matrix and scaling part of a step runs at raised priority: of the SIMD's two wavefronts
+            // the one that already holds its operands goes first, and reaches its next refill sooner
+            // (62.4 -> 61.9 us at T = 256, 60.3 -> 59.2 at T = 128; raising the first half of the step
+            // instead changes nothing).
+            __builtin_amdgcn_s_setprio(2);
 #pragma unroll
             for (int m = 0; m < nmb; ++m) {
                 {
@@ -371,6 +376,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
 #pragma unroll
                 for (int i = 0; i < 2; ++i)
                     asm volatile("" : "+v"(acc[i][m].x), "+v"(acc[i][m].y), "+v"(acc[i][m].z), "+v"(acc[i][m].w));
+            __builtin_amdgcn_s_setprio(0);
             ODSD_FENCE();
         };
         auto zero_acc = [&]() {
