@@ -4,7 +4,7 @@ It serves whole-block calls at the Qwen3-30B-A3B expert shape (hidden 2048, 128 
 intermediate 768) with 8 to 20 rows per expert on average; the stage entry points keep the
 two-launch plan.  The same hand-built routing goes through both, and through the CPU oracle:
 experts without rows, with exactly 16 / 17 / 32 / 33 rows (one and two token blocks, one and two
-passes) and one with 70 rows (three passes).  Replaces expert_forward_with_weights
+passes), one with 70 rows (three passes) and a heavily skewed routing (200 and 100 rows).  Replaces expert_forward_with_weights
 (demo/src/layers/mlp.py:227-230) inside the per-expert loop of qwen3_runner.py:303-380."""
 import numpy as np
 import pytest
@@ -60,6 +60,7 @@ CASES = [
     (128, {}),                                                   # 8 rows per expert on average
     (320, {}),                                                   # 20 on average: some experts take two passes
     (200, {0: 0, 1: 16, 2: 17, 3: 32, 4: 33, 5: 70, 6: 1, 127: 0}),
+    (256, {7: 200, 8: 100, 9: 0, 126: 49}),                      # heavy skew: up to seven passes over one expert's weights
 ]
 
 
