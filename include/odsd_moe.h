@@ -47,8 +47,9 @@ extern "C" {
 #endif
 
 /* 110: events / static forms of the whole block, KV store, paged and packed attention added (100: the MoE block)
- * 112: odsd_moe_shape.max_rows (was reserved, 0 keeps the old meaning), odsd_experts_one_launch */
-#define ODSD_VERSION 112
+ * 112: odsd_moe_shape.max_rows (was reserved, 0 keeps the old meaning), odsd_experts_one_launch
+ * 113: odsd_moe_static_init */
+#define ODSD_VERSION 113
 
 typedef enum odsd_status {
     ODSD_OK = 0,
@@ -308,6 +309,12 @@ int odsd_moe_forward_events(const odsd_moe_shape *s, const void *x, const void *
  * (two streams, two threads) race; run them one after the other.  Arguments and results are
  * those of odsd_moe_forward. */
 #define ODSD_STATIC_SCRATCH_BYTES (64u << 20)
+/* Set-up of the call below for the current device (no counterpart in the reference either): looks the
+ * array's device address up once and keeps it.  Call it once per device before the first
+ * odsd_moe_forward_static -- always before one that runs while a stream is being captured into a HIP
+ * graph, where the look-up must not happen.  (Without it the first odsd_moe_forward_static on a
+ * device does the look-up itself, which is fine outside capture.)  Allocates nothing. */
+int odsd_moe_static_init(void);
 int odsd_moe_forward_static(const odsd_moe_shape *s, const void *x, const void *norm_weight,
                             float eps, const void *gate_w, const uint64_t *table,
                             int32_t add_residual, float *out_f32, void *out_act,

@@ -15,7 +15,7 @@ def runtime() -> C.CDLL:
     """The HIP runtime already loaded into this process (by torch and by libodsd_moe.so)."""
     global _rt
     if _rt is None:
-        rt = C.CDLL("libamdhip64.so.7")
+        rt = _open_runtime()
         rt.hipEventCreate.argtypes = [C.POINTER(C.c_void_p)]
         rt.hipEventDestroy.argtypes = [C.c_void_p]
         rt.hipEventRecord.argtypes = [C.c_void_p, C.c_void_p]
@@ -23,6 +23,26 @@ def runtime() -> C.CDLL:
         rt.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
         _rt = rt
     return _rt
+
+
+def _open_runtime() -> C.CDLL:
+    """The copy of libamdhip64 that is mapped into this process, whatever its version suffix or
+    directory (a torch wheel may bring its own); failing that, the usual names in turn."""
+    try:
+        with open("/proc/self/maps") as f:
+            for line in f:
+                path = line.rsplit(None, 1)[-1]
+                if "libamdhip64.so" in path and path.startswith("/"):
+                    return C.CDLL(path)
+    except OSError:
+        pass
+    last = None
+    for name in ("libamdhip64.so", "libamdhip64.so.7", "libamdhip64.so.6", "libamdhip64.so.5"):
+        try:
+            return C.CDLL(name)
+        except OSError as e:
+            last = e
+    raise OSError(f"the HIP runtime (libamdhip64) is neither mapped into this process nor loadable: {last}")
 
 
 def _check(rc: int, what: str) -> None:

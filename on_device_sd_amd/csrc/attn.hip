@@ -115,7 +115,8 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
     const int L = varlen ? p.cu_k[seq + 1] - k_start : p.context_lens[seq];
     const int ql = varlen ? p.cu_q[seq + 1] - p.cu_q[seq] : (p.q_lens ? p.q_lens[seq] : 1);
     const int rows_total = ql * Gq;
-    if (L <= 0 || ql <= 0 || (int)blockIdx.y * 64 >= rows_total) return;
+    // (a sequence without cached keys still owns output rows: they are written as zeros below)
+    if (ql <= 0 || (int)blockIdx.y * 64 >= rows_total) return;
     const int row0 = ((int)blockIdx.y * 4 + wave) * 16;
     const bool wave_active = row0 < rows_total;
     const int D = p.KVH * HD;
@@ -130,9 +131,12 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
     const int tok = row_ok ? row / Gq : 0, hq = row_ok ? row % Gq : 0;
     V8 qf[NJ];
     int q0 = seq;
-    auto load_q = [&]() {
+    auto first_token = [&]() {
         if (varlen) q0 = p.cu_q[seq];
         else if (p.q_lens) q0 = attn_first_token(p.q_lens, seq);
+    };
+    auto load_q = [&]() {
+        first_token();
         const uint16_t *qp = (const uint16_t *)p.q + ((size_t)(q0 + tok) * p.H + kvh * Gq + hq) * HD + 8 * kq;
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
@@ -237,7 +241,7 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
     // (keys past the last one that any row of this workgroup attends are never visited: in a
     // prefill the early row groups stop long before the end of the sequence)
     const int last_tok = min(ql - 1, ((int)blockIdx.y * 64 + 63) / Gq);
-    const int k_end = min(L, L - ql + last_tok + 1);
+    const int k_end = max(0, min(L, L - ql + last_tok + 1));   // no visible key at all: no tiles, zeros out
     const int all_tiles = (k_end + 31) / 32;
     const int per_split = (all_tiles + p.splits - 1) / p.splits;
     const int t_begin = min(all_tiles, (int)blockIdx.z * per_split);
@@ -367,6 +371,8 @@ __global__ __launch_bounds__(256, 2) void paged_attn_kernel(const AttnParams p) 
         } else {
             tile(s0, no, no, it);
         }
+    } else {
+        first_token();     // the rows are still written (zeros): they need the sequence's first row
     }
 
     l_run += __shfl_xor(l_run, 16, ODSD_WAVE);
@@ -428,7 +434,6 @@ __global__ __launch_bounds__(256) void paged_attn_merge_kernel(const AttnParams 
     const bool varlen = p.cu_k != nullptr;
     const int ql = varlen ? p.cu_q[seq + 1] - p.cu_q[seq] : (p.q_lens ? p.q_lens[seq] : 1);
     const int rows_total = ql * Gq;
-    if ((varlen ? p.cu_k[seq + 1] - p.cu_k[seq] : p.context_lens[seq]) <= 0) return;
     // the sequence's first token: a chain of its own (a wavefront-wide sum over the query lengths),
     // started before the partial results are requested and by every lane of the wavefront
     int q0 = seq;

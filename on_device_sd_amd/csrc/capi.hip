@@ -169,6 +169,14 @@ static int scratch_for_current_device(void **out) {
     return ODSD_OK;
 }
 
+// Looks the array up for the current device.  Meant to be called once per device at set-up, so that
+// the call below does no runtime query at all on its hot path -- in particular none while a stream
+// is being captured into a HIP graph.
+extern "C" int odsd_moe_static_init(void) {
+    void *ws = nullptr;
+    return scratch_for_current_device(&ws);
+}
+
 extern "C" int odsd_moe_forward_static(const odsd_moe_shape *s, const void *x, const void *norm_weight,
                                        float eps, const void *gate_w, const uint64_t *table,
                                        int32_t add_residual, float *out_f32, void *out_act,

@@ -471,6 +471,9 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         ql = 1 if q_lens is None else int(np.asarray(q_lens)[i])
         q_seq = qf[q0:q0 + ql]
         q0 += ql
+        if L <= 0:
+            outs.append(torch.zeros((ql, H, HD)))              # nothing cached: an empty sum
+            continue
         table = np.asarray(block_tables[i]).tolist()
         slots = torch.tensor([table[p // block_size] * block_size + p % block_size for p in range(L)], dtype=torch.long)
         k_seq = kc.index_select(0, slots).view(L, num_kv_heads, HD).repeat_interleave(H // num_kv_heads, dim=1)
@@ -480,7 +483,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         o = F.scaled_dot_product_attention(q_seq.transpose(0, 1).unsqueeze(0), k_seq.transpose(0, 1).unsqueeze(0),
                                            v_seq.transpose(0, 1).unsqueeze(0), attn_mask=bias, dropout_p=0.0,
                                            is_causal=False, scale=scale)
-        outs.append(o.squeeze(0).transpose(0, 1))
+        # a query with no visible key (context_len < q_len) is an empty sum: zeros, as in varlen_attention
+        outs.append(torch.nan_to_num(o.squeeze(0).transpose(0, 1), nan=0.0))
     return torch.cat(outs, dim=0)
 
 

@@ -75,6 +75,12 @@ ATTN_CASES = [
     (torch.bfloat16, 32, 4, 128, 256, [(5000, 8)]),                                       # one long sequence: 19 key slices
     (torch.float16, 16, 8, 64, 64, [(3000, 4), (100, 4), (2977, 1)]),                     # slices with ragged ends, head_dim 64
     (torch.bfloat16, 32, 4, 128, 48, [(1500, 6), (700, 2)]),                              # block size not a multiple of the key tile
+    # fewer cached tokens than queries, and a sequence with nothing cached, in every position of the
+    # batch: the queries without a visible key are zeros, and the rows of the sequences after them
+    # must still land where they belong
+    (torch.bfloat16, 32, 4, 128, 16, [(300, 4), (3, 8), (0, 2), (40, 5)]),
+    (torch.float16, 8, 8, 64, 8, [(2, 6), (70, 3)]),
+    (torch.bfloat16, 16, 2, 128, 32, [(5000, 8), (0, 3), (1, 4)]),                        # with key slices (merge kernel)
 ]
 
 
@@ -84,7 +90,7 @@ def test_paged_attention_vs_oracle(dev, dtype, H, KVH, HD, bs, seqs):
     import on_device_sd_amd as odsd
     g = torch.Generator().manual_seed(H + HD + bs)
     decode = seqs[0][1] is None
-    n_blocks_per = [-(-L // bs) for L, _ in seqs]
+    n_blocks_per = [max(1, -(-L // bs)) for L, _ in seqs]
     total_blocks = sum(n_blocks_per) + 3
     perm = torch.randperm(total_blocks, generator=g).tolist()
     tables, at = [], 0
@@ -122,6 +128,8 @@ VARLEN_CASES = [
     (torch.float16, 8, 8, 64, [(130, 130), (64, 64)]),                      # no grouping, head_dim 64
     (torch.bfloat16, 16, 2, 128, [(40, 200), (5, 5), (64, 65)]),            # queries on top of earlier keys (chunked prefill)
     (torch.bfloat16, 32, 4, 128, [(1500, 1500)]),                           # one long sequence: many row groups, early key cut-off
+    (torch.bfloat16, 16, 2, 128, [(40, 10), (8, 3), (5, 0), (6, 6)]),       # more queries than keys: the first ones see nothing (zeros)
+    (torch.float16, 8, 8, 64, [(3, 1), (200, 130), (64, 64)]),
 ]
 
 

@@ -295,18 +295,75 @@ def test_gate_up_h_rows(dev, T, H, E, K, I, dtype):
         assert err <= 2e-3 * max(ref.abs().max().item(), 1e-3) + 1e-4, (e, err)
 
 
-def _clamped_reference(x, idx, w, experts, lim=65504.0):
-    """The oracle's per-expert loop with the two places where the device path holds fp16 values
-    made explicit: activations and h = silu(g) * u are clamped to +-65504."""
+def _clamped_reference(x, idx, w, experts, lim=65504.0, y_slices=0, tokens=None):
+    """The oracle's per-expert loop with the places where the device path holds fp16 values made
+    explicit: activations and h = silu(g) * u are clamped to +-65504, and so is an expert's output
+    row where the plan keeps it as fp16 -- y_slices = 1: the complete sum over the intermediate
+    features; 2: the sums over the two halves of the intermediate features, each clamped, then
+    added (the one-launch expert kernel); 0: fp32 partial sums, no clamp.  `tokens`: evaluate these
+    rows only."""
     xf = x.to(torch.float32).clamp(-lim, lim)
     T, K = idx.shape
+    toks = range(T) if tokens is None else tokens
     out = torch.zeros(T, xf.shape[1])
-    for k in range(K):
-        for t in range(T):
-            gw, uw, dw = experts[int(idx[t, k])].dequant()
+    cache = {}
+    for t in toks:
+        for k in range(K):
+            e = int(idx[t, k])
+            if e not in cache:
+                cache[e] = experts[e].dequant()
+            gw, uw, dw = cache[e]
             h = (torch.nn.functional.silu(xf[t] @ gw.T) * (xf[t] @ uw.T)).clamp(-lim, lim)
-            out[t] += float(w[t, k]) * (h @ dw.T)
+            if y_slices == 0:
+                y = h @ dw.T
+            else:
+                n = h.shape[0] // y_slices
+                y = sum((h[i * n:(i + 1) * n] @ dw[:, i * n:(i + 1) * n].T).clamp(-lim, lim) for i in range(y_slices))
+            out[t] += float(w[t, k]) * y
     return out
+
+
+SATURATING_Y_CASES = [
+    # T, H, E, K, I, w_mean, w_std, rows checked
+    (600, 256, 2, 2, 384, -0.5, 0.01, 600),     # 256-row tile kernel, complete sums as fp16
+    (40, 512, 4, 2, 384, -1.5, 0.01, 40),       # streaming kernel, unsplit reduction, complete sums as fp16
+    (128, 2048, 128, 8, 768, -0.5, 0.01, 12),   # one-launch expert kernel: two fp16 slices
+]
+
+
+@pytest.mark.parametrize("T,H,E,K,I,w_mean,w_std,n_check", SATURATING_Y_CASES)
+def test_expert_output_beyond_fp16_saturates_as_documented(dev, T, H, E, K, I, w_mean, w_std, n_check):
+    """Where a plan keeps an expert's output row as fp16 (an unsplit down projection, the one-launch
+    kernel's two slices) a value beyond +-65504 saturates -- the reference's bf16 would hold it.
+    Weights with a mean of -0.5 and more push per-expert outputs to 1e5 and beyond (far from any
+    LLM's): the block must then equal the oracle evaluated with the x, h AND y clamps, for the
+    plan the library reports for the shape, and differ from the unclamped oracle."""
+    import ctypes as C
+    from on_device_sd_amd import _lib
+    print("saturating expert outputs", T, H, E, K, I, w_mean, flush=True)
+    ops = _ops()
+    wg, bank, experts, x = _small_layer(dev, T, H, E, K, I, torch.bfloat16, seed=T + I, w_mean=w_mean, w_std=w_std)
+    lib = _lib.load()
+    shape = ops.make_shape(T, H, E, K, I, True, torch.bfloat16)
+    one_launch = lib.odsd_experts_one_launch(C.byref(shape))
+    splits = lib.odsd_w4_down_splits(C.byref(shape))
+    y_slices = 2 if one_launch == 1 else (1 if splits == 1 else 0)
+    assert y_slices > 0, "the case is meant to take a plan with fp16 expert outputs"
+    out = ops.moe_forward(x.to(dev), wg.to(dev), bank.table(), K, I, renorm=True)
+    lg = orc.router_logits(x, wg)
+    idx, w = orc.route(lg, K, True)
+    assert np.array_equal(out.idx.cpu().numpy(), idx)
+    got = out.out_f32.cpu()
+    assert torch.isfinite(got).all()
+    toks = list(range(n_check))
+    ref_c = _clamped_reference(x, idx, w, experts, y_slices=y_slices, tokens=toks)[:n_check]
+    ref_u = _clamped_reference(x, idx, w, experts, y_slices=0, tokens=toks)[:n_check]
+    assert (ref_u - ref_c).abs().max() > 100.0, "the case is meant to reach the clamp of y"
+    err = (got[:n_check] - ref_c).abs()
+    mx = err.max().item() / ref_c.abs().max().item()
+    print(f"  y slices {y_slices}: max error {mx:.2e} of max|clamped ref| = {ref_c.abs().max().item():.3e}; "
+          f"unclamped max {ref_u.abs().max().item():.3e}", flush=True)
+    assert mx <= 2e-3
 
 
 def test_outlier_activations(dev):

@@ -77,6 +77,18 @@ def test_oracle_paged_attention_against_plain_softmax():
                 ref = sum(wi * vc[slot(p), kvh * HD:(kvh + 1) * HD] for p, wi in enumerate(w)) / sum(w)
                 assert torch.allclose(out[q0 + j, h], ref.to(torch.float32), atol=1e-5)
         q0 += ql
+    # fewer cached tokens than queries: query j sees positions 0 .. L - ql + j, the first ql - L
+    # queries see nothing and are zeros; the others are a scalar softmax over what they see
+    short = orc.paged_attention(q, kc, vc, tables, [2, 0], [4, 1], KVH, bs, 0.3)
+    assert torch.equal(short[:2], torch.zeros(2, H, HD)) and torch.equal(short[4], torch.zeros(H, HD))
+    slot = lambda p: tables[0][p // bs] * bs + p % bs
+    for j in (2, 3):
+        for h in range(H):
+            kvh = h // (H // KVH)
+            sc = [float(q[j, h] @ kc[slot(p), kvh * HD:(kvh + 1) * HD]) * 0.3 for p in range(j - 1)]
+            w = np.exp(np.array(sc) - max(sc))
+            ref = sum(wi * vc[slot(p), kvh * HD:(kvh + 1) * HD] for p, wi in enumerate(w)) / w.sum()
+            assert torch.allclose(short[j, h], ref.to(torch.float32), atol=1e-5)
     dec = orc.paged_attention(q[:2], kc, vc, tables, lens, None, KVH, bs, 0.3)
     one = orc.paged_attention(q[:2], kc, vc, tables, lens, [1, 1], KVH, bs, 0.3)
     assert torch.equal(dec, one)
@@ -113,6 +125,16 @@ def test_oracle_varlen_attention_pins():
             w = np.exp(np.array(sc) - max(sc))
             ref = sum(wi * v2[p, kvh] for p, wi in enumerate(w)) / w.sum()
             assert torch.allclose(o2[j, h], ref.to(torch.float32), atol=1e-5)
+    # (b') 4 queries on 2 keys: queries 0 and 1 see no key (zeros), query j >= 2 sees keys 0 .. j - 2
+    o3 = orc.varlen_attention(q[:4], k[:2], v[:2], [0, 4], [0, 2], 0.4)
+    assert torch.equal(o3[:2], torch.zeros(2, H, HD))
+    for j in (2, 3):
+        for h in range(H):
+            kvh = h // (H // KVH)
+            sc = [float(q[j, h] @ k[p, kvh]) * 0.4 for p in range(j - 1)]
+            w = np.exp(np.array(sc) - max(sc))
+            ref = sum(wi * v[p, kvh] for p, wi in enumerate(w)) / w.sum()
+            assert torch.allclose(o3[j, h], ref.to(torch.float32), atol=1e-5)
     # (c) the same prefill through a cache with 4-token blocks in scrambled order
     bs = 4
     tables, kc, vc, nxt = [], torch.zeros(8 * bs, KVH * HD), torch.zeros(8 * bs, KVH * HD), [5, 2, 7, 0, 3, 6, 1, 4]

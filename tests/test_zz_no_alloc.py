@@ -62,3 +62,56 @@ def test_static_scratch_matches_workspace_call(dev):
             assert torch.equal(got[name].view(torch.uint8), ref[name].view(torch.uint8)), \
                 f"T={T}: {name} differs between the static-scratch call and the workspace call"
         assert int(ref["counts"].sum()) == T * K and torch.isfinite(ref["out_f32"]).all()
+
+
+def test_static_scratch_call_under_graph_capture(dev):
+    """The use the entry point is offered for: after odsd_moe_static_init() the call is captured into
+    a HIP graph (nothing may allocate or query the runtime there) and replayed several times, with
+    eager work and synchronisations of the program's own between the replays; every replay must give
+    the bits of the eager workspace call."""
+    from on_device_sd_amd import _lib
+    lib = _lib.load()
+    T, H, E, K, I = 48, 512, 16, 4, 512
+    print("no-alloc entry point under graph capture: T", T, flush=True)
+    gate, bank, x, norm = _layer(dev, T, H, E, K, I, 21)
+    table = bank.table()
+    shape = _lib.MoeShape(T, H, E, K, I, 1, _lib.DT_BF16, 0)
+    _lib.check(lib.odsd_moe_static_init(), "odsd_moe_static_init")
+    ref = _run(lib, False, shape, x, norm, gate, table, dev)
+    out_f32 = torch.zeros(T, H, dtype=torch.float32, device=dev)
+    out_act = torch.zeros(T, H, dtype=torch.bfloat16, device=dev)
+    idx = torch.zeros(T, K, dtype=torch.int32, device=dev)
+    x_in = x.clone()
+
+    def call():
+        _lib.check(lib.odsd_moe_forward_static(
+            C.byref(shape), x_in.data_ptr(), norm.data_ptr(), 1e-6, gate.data_ptr(), table.data_ptr(), 1,
+            out_f32.data_ptr(), out_act.data_ptr(), idx.data_ptr(), None, None, None, None, None, None,
+            torch.cuda.current_stream().cuda_stream), "odsd_moe_forward_static")
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call()                                   # warm-up on the capture stream, outside capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated(dev)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    assert torch.cuda.memory_allocated(dev) == before, "the captured call allocated device memory"
+    for rep in range(4):
+        out_f32.fill_(float("nan")); out_act.zero_(); idx.fill_(-1)
+        if rep == 2:                             # other inputs through the same graph, then the first ones again
+            x_in.copy_(torch.flip(x, dims=[0]))
+        elif rep == 3:
+            x_in.copy_(x)
+        graph.replay()
+        torch.cuda.synchronize()
+        if rep == 2:
+            assert torch.equal(idx, torch.flip(ref["idx"], dims=[0]))
+            continue
+        for name, got in (("out_f32", out_f32), ("out_act", out_act), ("idx", idx)):
+            assert torch.equal(got.view(torch.uint8), ref[name].view(torch.uint8)), f"replay {rep}: {name} differs"
+        # eager work of the program's own on the shared scratch between the replays
+        _run(lib, True, _lib.MoeShape(20, H, E, K, I, 1, _lib.DT_BF16, 0), x[:20].contiguous(), norm, gate, table, dev)
