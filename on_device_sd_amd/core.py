@@ -7,8 +7,9 @@ code written against the reference works unchanged on top of this runner.
 """
 from __future__ import annotations
 
+from collections.abc import Set as AbstractSet
 from dataclasses import dataclass, field
-from typing import Any, Dict, NamedTuple, Optional, Set, Tuple
+from typing import Any, Callable, Dict, NamedTuple, Optional, Set, Tuple
 
 import torch
 
@@ -24,11 +25,55 @@ class ExpertID(NamedTuple):
         return f"L{self.layer_idx}_E{self.expert_idx}"
 
 
+class LazyExpertSet(AbstractSet):
+    """The activated set of a routing result, read from the device when it is first looked at.
+
+    The reference builds the set inside route_experts with a blocking device-to-host copy
+    (qwen3_runner.py:110-112), whether or not anybody reads it.  Here the copy of the per-expert
+    counts is started by route_experts and waited for on first use -- iteration, ``in``, ``len``,
+    comparison or a set operation (which give plain sets) -- so a step whose placement never looks
+    at the set (every expert resident) never stops the host.  It compares equal to a ``set`` with
+    the same members."""
+
+    def __init__(self, fetch: Callable[[], Set["ExpertID"]]):
+        self._fetch: Optional[Callable[[], Set["ExpertID"]]] = fetch
+        self._set: Optional[Set["ExpertID"]] = None
+
+    def _get(self) -> Set["ExpertID"]:
+        if self._set is None:
+            self._set = self._fetch()
+            self._fetch = None
+        return self._set
+
+    @property
+    def resolved(self) -> bool:
+        """True once the set has been read from the device."""
+        return self._set is not None
+
+    def __contains__(self, item) -> bool:
+        return item in self._get()
+
+    def __iter__(self):
+        return iter(self._get())
+
+    def __len__(self) -> int:
+        return len(self._get())
+
+    @classmethod
+    def _from_iterable(cls, it):
+        return set(it)
+
+    def __repr__(self) -> str:
+        return f"LazyExpertSet({self._set!r})" if self._set is not None else "LazyExpertSet(<not read yet>)"
+
+
 @dataclass
 class RoutingResult:
     """What route_experts returns (model_runner.py:14-27).
 
     topk_indices [T, K] int64 in descending-score order, topk_scores [T, K] float32.
+    ``activated_expert_ids`` of a result that route_experts made is a ``LazyExpertSet``: the set
+    of unique selected experts, read from the device at first use.
     ``dispatch`` is an optional cache of the device-side dispatch arrays that
     route_experts already produced; forward_moe recomputes them when it is absent
     (for example on a hand-built RoutingResult).  ``x_f16`` is the fp16 copy of the routed
@@ -47,13 +92,26 @@ class RoutingResult:
     # the routed tensor itself: while the routing result lives, its storage cannot be handed to
     # another tensor, so the address in x_tag keeps meaning "that tensor"
     x_src: Optional[torch.Tensor] = field(default=None, repr=False, compare=False)
-    # the largest per-expert pair count, read on the host together with the activated set
-    # (0: not known); forward_moe hands it to the library with the dispatch arrays it belongs to
+    # the largest per-expert pair count (0: not known); forward_moe hands it to the library with
+    # the dispatch arrays it belongs to.  route_experts leaves it 0 and fills ``counts_host``.
     max_rows: int = field(default=0, repr=False, compare=False)
+    # route_experts: the per-expert counts on their way to the host (an object with ``ready`` and
+    # ``get()``); read by whoever first needs the activated set
+    counts_host: Optional[Any] = field(default=None, repr=False, compare=False)
 
     @property
     def top_k(self) -> int:
         return self.topk_indices.shape[-1]
+
+    def known_max_rows(self) -> int:
+        """The largest per-expert pair count if the host already has it, else 0 -- never waits."""
+        if self.max_rows > 0:
+            return self.max_rows
+        c = self.counts_host
+        if c is not None and c.ready:
+            counts = c.get()
+            return int(counts.max()) if counts.size else 0
+        return 0
 
 
 @dataclass

@@ -6,7 +6,10 @@ its optional ``src_index`` folds in the ``index_select`` of the draft tokens tha
 does first (``attention.py:222-228``).  ``SequenceSlots`` and ``build_verify_context`` are the
 host bookkeeping that produces the slot list and the rest of the verify context, with the fields
 and arithmetic of ``SequenceState`` / ``PagedKVCache.get_verify_context``
-(``demo/src/memory/paged_kv_cache.py:127-207, :542-580``); they are plain Python and need no GPU.
+(``demo/src/memory/paged_kv_cache.py:127-207, :542-580``); ``build_prefill_context`` and
+``build_decode_context`` are the other two forms (``_get_prefill_context`` / ``_get_decode_context``,
+``:484-540``) and ``get_attention_context`` picks between them as ``:463-482`` does.  They are plain
+Python and need no GPU; ``attention_for_context`` runs the attention kernel that fits a context.
 """
 from __future__ import annotations
 
@@ -71,25 +74,30 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     dt = {torch.bfloat16: _lib.DT_BF16, torch.float16: _lib.DT_F16}.get(q.dtype)
     if dt is None:
         raise TypeError("paged attention takes bfloat16 or float16")
-    tables = context["block_tables"].to(torch.int32).contiguous()
-    lens = context["context_lens"].to(torch.int32).contiguous()
+    tables = context["block_tables"].to(device=q.device, dtype=torch.int32).contiguous()
+    lens = context["context_lens"].to(device=q.device, dtype=torch.int32).contiguous()
     q_lens = context.get("verify_query_lens")
-    if q_lens is not None:
-        q_lens = q_lens.to(torch.int32).contiguous()
     n_seqs = lens.numel()
     out = torch.empty_like(q)
     if n_seqs == 0 or n_tokens == 0:
         return out
     scale = head_dim ** -0.5 if softmax_scale is None else softmax_scale
     lib = _lib.load()
-    mq = max_q_len or n_tokens
+    # max_q_len sizes the launch: rows of a sequence beyond it would not be computed.  Without the
+    # caller's bound n_tokens is used (no sequence can hold more); a bound that came with the context
+    # (the builders below know the lengths on the host) is taken; lengths that are readable without a
+    # device synchronisation are checked against an explicit bound.
+    mq = max_q_len or context.get("max_query_len") or n_tokens
+    if max_q_len and q_lens is not None and not q_lens.is_cuda and q_lens.numel() and int(q_lens.max()) > max_q_len:
+        raise ValueError(f"max_q_len={max_q_len} is below the longest query ({int(q_lens.max())} tokens)")
     nbytes = lib.odsd_paged_attention_workspace_bytes(n_seqs, mq, num_heads, num_kv_heads, head_dim, block_size,
                                                       tables.shape[1])
     if nbytes == 0:
         raise _lib.OdsdError("paged attention: unsupported shape (head_dim 64 or 128, heads a multiple of KV heads)")
     ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+    q_lens_dev = None if q_lens is None else q_lens.to(device=q.device, dtype=torch.int32).contiguous()
     _lib.check(lib.odsd_paged_attention(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), tables.data_ptr(),
-                                        lens.data_ptr(), None if q_lens is None else q_lens.data_ptr(), n_seqs,
+                                        lens.data_ptr(), None if q_lens_dev is None else q_lens_dev.data_ptr(), n_seqs,
                                         mq, num_heads, num_kv_heads, head_dim, block_size,
                                         tables.shape[1], k_cache.numel() // D, scale, dt, out.data_ptr(),
                                         ws.data_ptr(), nbytes, torch.cuda.current_stream().cuda_stream),
@@ -181,6 +189,64 @@ def build_verify_context(sequences: Dict[int, SequenceSlots], seq_ids: Sequence[
         max_num_blocks = max(max_num_blocks, len(st.block_table))
     tables = [sequences[s].get_block_table(max_num_blocks) for s in seq_ids]
     mk = lambda v: torch.tensor(v, dtype=torch.int32, device=device)
+    # (max_query_len is this build's addition: the host already knows it, and the attention launch is
+    # sized by it)
     return {"slot_mapping": mk(slot_mapping), "context_lens": mk(context_lens),
             "block_tables": mk(tables).reshape(len(seq_ids), max_num_blocks),
-            "verify_query_lens": mk(verify_query_lens), "verify_q_indices": mk(verify_q_indices)}
+            "verify_query_lens": mk(verify_query_lens), "verify_q_indices": mk(verify_q_indices),
+            "max_query_len": max(verify_query_lens, default=0)}
+
+
+def build_prefill_context(sequences: Dict[int, SequenceSlots], seq_ids: Sequence[int], device="cuda") -> Dict:
+    """``PagedKVCache._get_prefill_context`` (paged_kv_cache.py:484-511): every token of every
+    sequence is new -- packed one sequence after the other, with its slot -- and queries and keys
+    have the same lengths."""
+    cu = [0]
+    slot_mapping: List[int] = []
+    longest = 0
+    for seq_id in seq_ids:
+        st = sequences[seq_id]
+        n = st.num_tokens
+        cu.append(cu[-1] + n)
+        longest = max(longest, n)
+        slot_mapping.extend(st.get_slot_mapping(0, n))
+    mk = lambda v: torch.tensor(v, dtype=torch.int32, device=device)
+    return {"slot_mapping": mk(slot_mapping), "cu_seqlens_q": mk(cu), "cu_seqlens_k": mk(cu),
+            "max_seqlen_q": longest, "max_seqlen_k": longest}
+
+
+def build_decode_context(sequences: Dict[int, SequenceSlots], seq_ids: Sequence[int], device="cuda") -> Dict:
+    """``PagedKVCache._get_decode_context`` (paged_kv_cache.py:513-540): one new token per sequence,
+    the last one; its slot, the sequence's length including it, and the padded block tables."""
+    slot_mapping: List[int] = []
+    context_lens: List[int] = []
+    max_num_blocks = 0
+    for seq_id in seq_ids:
+        st = sequences[seq_id]
+        slot_mapping.extend(st.get_slot_mapping(st.num_tokens - 1, 1))
+        context_lens.append(st.num_tokens)
+        max_num_blocks = max(max_num_blocks, len(st.block_table))
+    tables = [sequences[s].get_block_table(max_num_blocks) for s in seq_ids]
+    mk = lambda v: torch.tensor(v, dtype=torch.int32, device=device)
+    return {"slot_mapping": mk(slot_mapping), "context_lens": mk(context_lens),
+            "block_tables": mk(tables).reshape(len(seq_ids), max_num_blocks), "max_query_len": 1}
+
+
+def get_attention_context(sequences: Dict[int, SequenceSlots], seq_ids: Sequence[int], is_prefill: bool,
+                          device="cuda") -> Dict:
+    """``PagedKVCache.get_attention_context`` (paged_kv_cache.py:463-482)."""
+    return build_prefill_context(sequences, seq_ids, device) if is_prefill \
+        else build_decode_context(sequences, seq_ids, device)
+
+
+def attention_for_context(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_cache: torch.Tensor,
+                          v_cache: torch.Tensor, context: Dict, num_kv_heads: int, block_size: int,
+                          softmax_scale: Optional[float] = None) -> torch.Tensor:
+    """The branch of ``Qwen3Attention.forward`` after the KV store (attention.py:229-282): a prefill
+    context (it carries ``cu_seqlens_q``) attends the step's own packed k / v, a decode or verify
+    context reads the paged cache.  q: [n_tokens, num_heads, head_dim]; k, v: [n_tokens,
+    num_kv_heads, head_dim] (unused for decode / verify)."""
+    if "cu_seqlens_q" in context:
+        return varlen_attention(q, k, v, context["cu_seqlens_q"], context["cu_seqlens_k"],
+                                context["max_seqlen_q"], context["max_seqlen_k"], softmax_scale)
+    return paged_attention(q, k_cache, v_cache, context, num_kv_heads, block_size, softmax_scale)

@@ -12,11 +12,17 @@ device-to-host copy of the counts per key tells the host where each activation's
 ``build_prefill_placement`` mirrors ``model_runner_utils.py:56-79``: every activated expert is
 looked up in the shared set, the cache and the loader (in that order).  The cache and the loader
 are the engine's objects; only their methods named below are used.
+
+``build_draft_placement`` mirrors ``model_runner_utils.py:82-151``, the placement of a speculative
+draft step: activated experts that are not resident are either kept exact (the scheduler's
+``select_cpu_experts`` picks, at most ``top_c``) or replaced by a resident expert
+(``select_gpu_substitutes``); the substitutes' parameters are added to the placement and the
+``substitution_map`` tells the executor whose weights serve whose tokens.
 """
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Any, Dict, List
+from typing import Any, Dict, List, Set
 
 import torch
 
@@ -93,3 +99,67 @@ def build_prefill_placement(routing_result: RoutingResult, expert_cache: Any,
         if params is not None:
             gpu[expert_id.expert_idx] = params
     return ExpertPlacement(gpu_expert_params=gpu, cpu_expert_params={}, routing_result=routing_result)
+
+
+def build_draft_placement(routing_result: RoutingResult, expert_cache: Any, parameter_loader: Any,
+                          draft_scheduler: Any, *, top_c: int, num_experts: int,
+                          gpu_device: Any = "gpu", cpu_device: Any = "cpu") -> ExpertPlacement:
+    """Placement of a draft step (model_runner_utils.py:82-151), decision for decision:
+
+    1. the activated experts with a resident copy (shared set, cache, loader) are available;
+    2. of the others, the scheduler's ``select_cpu_experts(activations, top_c)`` names up to
+       ``top_c`` that are to be computed with their own weights: their parameters are asked of the
+       loader with ``device=cpu_device`` and go to ``cpu_expert_params``;
+    3. what is left is handed to ``select_gpu_substitutes(requested_experts, cached_experts,
+       all_experts)``; its answer becomes ``substitution_map`` (expert index -> expert index), and
+       the substitutes' resident parameters are put into ``gpu_expert_params``.
+
+    This runner has no CPU expert path: every bundle of either dict must be a W4 bundle in HBM (a
+    loader that keeps its off-cache experts as W4 bundles in a second bank can serve step 2), and
+    ``forward_moe`` raises ``TypeError`` for anything else.  A loader that answers ``None`` leaves
+    the expert out and the executor skips its pairs, as the reference does (qwen3_runner.py:330-333);
+    with ``top_c == 0`` every non-resident expert is substituted."""
+    layer = routing_result.layer_idx
+    activated: Set[ExpertID] = set(routing_result.activated_expert_ids)
+    resident: Dict[ExpertID, Any] = {}
+    for expert_id in activated:
+        params = _resident_params(expert_id, expert_cache, parameter_loader, gpu_device)
+        if params is not None:
+            resident[expert_id] = params
+    available: Set[ExpertID] = set(resident)
+    missing = activated - available
+
+    exact_ids: Set[ExpertID] = set()
+    if missing and top_c > 0:
+        acts = build_layer_activations(routing_result, num_experts)
+        candidates = [a for a in acts.activations if a.expert_id in missing]
+        if candidates:
+            exact_ids = set(draft_scheduler.select_cpu_experts(
+                LayerExpertActivations(layer_idx=acts.layer_idx, activations=candidates,
+                                       routing_scores=acts.routing_scores), top_c))
+
+    needs_substitution = activated - available - exact_ids
+    all_layer_experts = [ExpertID(layer, i) for i in range(num_experts)]
+    chosen = draft_scheduler.select_gpu_substitutes(
+        requested_experts=sorted(needs_substitution, key=lambda x: x.expert_idx),
+        cached_experts=set(available), all_experts=all_layer_experts)
+
+    gpu: Dict[int, Any] = {}
+    cpu: Dict[int, Any] = {}
+    for expert_id in sorted(activated, key=lambda x: x.expert_idx):
+        if expert_id in exact_ids:
+            params = parameter_loader.get_expert_params(expert_id, device=cpu_device)
+            if params is not None:
+                cpu[expert_id.expert_idx] = params
+            continue
+        if expert_id in resident:
+            gpu[expert_id.expert_idx] = resident[expert_id]
+    for sub_id in chosen.values():        # a substitute need not be activated itself
+        params = resident.get(sub_id)
+        if params is None:
+            params = _resident_params(sub_id, expert_cache, parameter_loader, gpu_device)
+        if params is not None:
+            gpu[sub_id.expert_idx] = params
+    return ExpertPlacement(gpu_expert_params=gpu, cpu_expert_params=cpu,
+                           substitution_map={o.expert_idx: s_.expert_idx for o, s_ in chosen.items()},
+                           routing_result=routing_result)

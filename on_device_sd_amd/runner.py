@@ -28,12 +28,40 @@ from typing import Dict, List, Optional
 import torch
 
 from . import ops
-from .core import (AttentionOutput, ExpertID, ExpertPlacement, LayerOutput, MoEConfig,
+from .core import (AttentionOutput, ExpertID, ExpertPlacement, LayerOutput, LazyExpertSet, MoEConfig,
                    RoutingResult)
 from .w4 import W4ExpertBank, W4ExpertParams, build_table
 
 
+class _CountsInFlight:
+    """The per-expert counts of one routing result on their way to pinned host memory.  ``get()``
+    waits for the copy (first call only); if the landing buffer has been handed to a later routing
+    result in the meantime, the counts are fetched from the device arrays instead."""
+    __slots__ = ("_runner", "_slot", "_gen", "_device_counts", "_np")
+
+    def __init__(self, runner, slot, gen, device_counts):
+        self._runner, self._slot, self._gen, self._device_counts, self._np = runner, slot, gen, device_counts, None
+
+    @property
+    def ready(self) -> bool:
+        return self._np is not None
+
+    def get(self):
+        if self._np is None:
+            r = self._runner
+            if r._ring_gen[self._slot] == self._gen:
+                r._ring_events[self._slot].synchronize()
+                if r._ring_gen[self._slot] == self._gen:
+                    self._np = r._ring_np[self._slot].copy()
+            if self._np is None:
+                self._np = self._device_counts.cpu().numpy()
+            self._runner = self._device_counts = None
+        return self._np
+
+
 class W4MoERunner:
+    COUNTS_RING = 64      # routing results whose counts can be in flight before a read falls back to a device copy
+
     def __init__(self, config: MoEConfig, gate_weights: List[torch.Tensor],
                  banks: List[W4ExpertBank], norm_weights: Optional[List[torch.Tensor]] = None):
         """gate_weights[l]: [E, H] router weight of layer l (model dtype);
@@ -46,12 +74,15 @@ class W4MoERunner:
         self.norm_weights = None if norm_weights is None else [
             n.to(device=self.device, dtype=self.dtype).contiguous() for n in norm_weights]
         self._table_cache: Dict[tuple, tuple] = {}
-        # host side of the hop between routing and execution: a pinned landing buffer for the E
-        # counts, an event to wait for just that copy, and the ExpertID objects made once
+        # host side of the hop between routing and execution: a ring of pinned landing buffers for
+        # the E counts (one per routing result in flight), an event per buffer to wait for just
+        # that copy, and the ExpertID objects made once
         E = config.num_experts
-        self._counts_host = torch.empty(E, dtype=torch.int32, pin_memory=True)
-        self._counts_np = self._counts_host.numpy()
-        self._counts_event = torch.cuda.Event()
+        self._ring = torch.empty(self.COUNTS_RING, E, dtype=torch.int32, pin_memory=True)
+        self._ring_np = self._ring.numpy()
+        self._ring_events = [torch.cuda.Event() for _ in range(self.COUNTS_RING)]
+        self._ring_gen = [0] * self.COUNTS_RING
+        self._ring_next = 0
         self._expert_ids = [[ExpertID(l, e) for e in range(E)] for l in range(len(banks))]
 
     # -- ModelRunner interface -----------------------------------------------------------------
@@ -66,19 +97,23 @@ class W4MoERunner:
         flat = hidden_states.reshape(-1, hidden_states.shape[-1])
         _, w, idx64, x16, disp = ops.route_dispatch(flat, self.gate_weights[layer_idx],
                                                     cfg.num_experts_per_token, cfg.norm_topk_prob)
-        # the engine reads the activated set on the host between routing and execution
-        # (qwen3_runner.py:110-112): one asynchronous copy of the E counts into pinned memory,
-        # and a wait for that copy alone
-        self._counts_host.copy_(disp.counts, non_blocking=True)
-        self._counts_event.record()
-        self._counts_event.synchronize()
+        # The engine reads the activated set on the host between routing and execution
+        # (qwen3_runner.py:110-112).  The E counts start their way to pinned memory here, by one
+        # asynchronous copy with an event of its own; the host waits for that event when the set
+        # (or the largest count) is first looked at -- a placement that takes every expert as
+        # resident never looks, and the step then runs without a host stop.
+        slot = self._ring_next
+        self._ring_next = (slot + 1) % self.COUNTS_RING
+        self._ring_gen[slot] += 1
+        self._ring[slot].copy_(disp.counts, non_blocking=True)
+        self._ring_events[slot].record()
+        counts = _CountsInFlight(self, slot, self._ring_gen[slot], disp.counts)
         ids = self._expert_ids[layer_idx] if layer_idx < len(self._expert_ids) else \
             [ExpertID(layer_idx, e) for e in range(cfg.num_experts)]
-        activated = set(map(ids.__getitem__, self._counts_np.nonzero()[0].tolist()))
+        activated = LazyExpertSet(lambda: set(map(ids.__getitem__, counts.get().nonzero()[0].tolist())))
         return RoutingResult(layer_idx=layer_idx, topk_indices=idx64, topk_scores=w,
                              activated_expert_ids=activated, dispatch=disp, x_f16=x16,
-                             x_tag=_tensor_tag(flat), x_src=hidden_states,
-                             max_rows=int(self._counts_np.max()) if self._counts_np.size else 0)
+                             x_tag=_tensor_tag(flat), x_src=hidden_states, counts_host=counts)
 
     def forward_moe(self, layer_idx: int, attn_output: AttentionOutput,
                     expert_placement: ExpertPlacement) -> torch.Tensor:
@@ -171,7 +206,7 @@ class W4MoERunner:
         _, out = ops.experts_w4(x16, table, idx, scores, disp,
                                 self.config.moe_intermediate_size, flat.dtype, residual=res,
                                 want_f32=False, want_act=True,
-                                max_rows=routing.max_rows if routing.dispatch is not None else 0)
+                                max_rows=routing.known_max_rows() if routing.dispatch is not None else 0)
         return out.view(shape)
 
 

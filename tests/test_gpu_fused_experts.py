@@ -204,4 +204,12 @@ def test_max_rows_statement_takes_the_two_launch_plan(dev, layer):
     wg = (torch.randn(E, H, generator=g) * 0.02).to(torch.bfloat16)
     runner = odsd.W4MoERunner(cfg, [wg.to(dev)], [bank])
     routing = runner.route_experts(0, x.to(dev))
-    assert routing.max_rows == int(routing.dispatch.counts.max().item()) > 0
+    # nothing has looked at the activated set yet: the host has not waited, the count is not known
+    assert not routing.activated_expert_ids.resolved and routing.known_max_rows() == 0
+    n_act = len(routing.activated_expert_ids)                  # the first look waits for the counts
+    assert routing.activated_expert_ids.resolved and n_act == int((routing.dispatch.counts > 0).sum())
+    assert routing.known_max_rows() == int(routing.dispatch.counts.max().item()) > 0
+    # more routing results than the runner has landing buffers: the oldest one still answers
+    old = runner.route_experts(0, x.to(dev))
+    later = [runner.route_experts(0, x.to(dev)) for _ in range(runner.COUNTS_RING + 3)]
+    assert set(old.activated_expert_ids) == set(later[-1].activated_expert_ids) == set(routing.activated_expert_ids)

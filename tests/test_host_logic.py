@@ -110,6 +110,56 @@ def test_prefill_placement_lookup_order_without_gpu():
     assert ("loader", 3) not in calls and ("loader", 4) not in calls and ("loader", 5) in calls
 
 
+def test_draft_placement_decisions_without_gpu():
+    """build_draft_placement with top_c = 0 is host logic (model_runner_utils.py:82-151): resident
+    experts are kept, the others are handed to the scheduler for substitution, the substitutes'
+    parameters are forced into the GPU dict even when they were not activated, and the map is
+    expressed in expert indices."""
+    from on_device_sd_amd.core import ExpertID, RoutingResult
+    from on_device_sd_amd.placement import build_draft_placement
+    GPU = object()
+    resident = {0, 2, 7}                    # experts the loader holds on the GPU
+
+    class Loader:
+        def is_shared_expert(self, eid): return False
+        def get_expert_params(self, eid, device=None):
+            assert device is GPU
+            return {"who": eid.expert_idx} if eid.expert_idx in resident else None
+
+    class Cache:
+        def is_cached(self, eid): return False
+
+    seen = {}
+
+    class Scheduler:
+        def select_cpu_experts(self, activations, top_c):
+            raise AssertionError("top_c = 0: the scheduler is not asked for exact experts")
+        def select_gpu_substitutes(self, requested_experts, cached_experts, all_experts):
+            seen.update(requested=list(requested_experts), cached=set(cached_experts), n_all=len(all_experts))
+            # expert 7 is resident but was not activated: the scheduler may only pick from `cached`
+            return {r: ExpertID(r.layer_idx, 2) for r in requested_experts}
+
+    rr = RoutingResult(layer_idx=1, topk_indices=torch.tensor([[0, 3], [2, 5]]), topk_scores=torch.ones(2, 2),
+                       activated_expert_ids={ExpertID(1, e) for e in (0, 2, 3, 5)})
+    pl = build_draft_placement(rr, Cache(), Loader(), Scheduler(), top_c=0, num_experts=8, gpu_device=GPU)
+    assert [e.expert_idx for e in seen["requested"]] == [3, 5] and seen["n_all"] == 8
+    assert seen["cached"] == {ExpertID(1, 0), ExpertID(1, 2)}
+    assert pl.substitution_map == {3: 2, 5: 2}
+    assert {e: p["who"] for e, p in pl.gpu_expert_params.items()} == {0: 0, 2: 2}
+    assert pl.cpu_expert_params == {} and pl.routing_result is rr
+
+    # a substitute that was not activated itself is fetched and added
+    class Scheduler2(Scheduler):
+        def select_gpu_substitutes(self, requested_experts, cached_experts, all_experts):
+            return {r: ExpertID(r.layer_idx, 7) for r in requested_experts}
+    pl2 = build_draft_placement(rr, Cache(), Loader(), Scheduler2(), top_c=0, num_experts=8, gpu_device=GPU)
+    assert pl2.substitution_map == {3: 7, 5: 7} and set(pl2.gpu_expert_params) == {0, 2, 7}
+    # everything resident: nothing is requested, nothing substituted
+    resident |= {3, 5}
+    pl3 = build_draft_placement(rr, Cache(), Loader(), Scheduler(), top_c=4, num_experts=8, gpu_device=GPU)
+    assert pl3.substitution_map == {} and set(pl3.gpu_expert_params) == {0, 2, 3, 5}
+
+
 def test_lru_strategy_and_cache_capacity():
     from on_device_sd_amd.cache import LRUStrategy, cache_capacity
     ids = [odsd.ExpertID(0, e) for e in range(4)]

@@ -4,7 +4,8 @@ import numpy as np
 import torch
 
 from oracle import moe_oracle as orc
-from on_device_sd_amd.kv import SequenceSlots, build_verify_context
+from on_device_sd_amd.kv import (SequenceSlots, build_decode_context, build_prefill_context, build_verify_context,
+                                  get_attention_context)
 
 
 def test_slot_mapping_by_hand():
@@ -33,11 +34,39 @@ def test_verify_context_matches_the_oracle_and_a_hand_case():
     assert ctx["verify_query_lens"].tolist() == [4, 1, 5]
     assert ctx["verify_q_indices"].tolist() == [1, 2, 3, 6, 7, 8, 9]
     assert ctx["block_tables"].tolist() == [[3, 0, -1], [1, -1, -1], [6, 4, 5]]
-    assert all(t.dtype == torch.int32 for t in ctx.values())
+    assert all(t.dtype == torch.int32 for t in ctx.values() if isinstance(t, torch.Tensor))
+    assert ctx["max_query_len"] == 5
     ref = orc.verify_context([dict(block_table=seqs[i].block_table, num_tokens=seqs[i].num_tokens,
                                    draft_start_num_tokens=seqs[i].draft_start_num_tokens) for i in (5, 9, 2)], 4)
     for k, v in ref.items():
         assert ctx[k].tolist() == v, k
+
+
+def test_prefill_and_decode_contexts_by_hand():
+    """The other two context forms of PagedKVCache (paged_kv_cache.py:484-540), worked by hand."""
+    seqs = {
+        1: SequenceSlots(block_size=4, block_table=[2, 5], num_tokens=6),
+        4: SequenceSlots(block_size=4, block_table=[0], num_tokens=3),
+        7: SequenceSlots(block_size=4, block_table=[9, 1, 3], num_tokens=9),
+    }
+    pre = build_prefill_context(seqs, [1, 4, 7], device="cpu")
+    assert pre["cu_seqlens_q"].tolist() == [0, 6, 9, 18] and pre["cu_seqlens_k"].tolist() == [0, 6, 9, 18]
+    assert pre["max_seqlen_q"] == 9 and pre["max_seqlen_k"] == 9
+    assert pre["slot_mapping"].tolist() == [8, 9, 10, 11, 20, 21, 0, 1, 2, 36, 37, 38, 39, 4, 5, 6, 7, 12]
+    dec = build_decode_context(seqs, [7, 1, 4], device="cpu")
+    assert dec["slot_mapping"].tolist() == [12, 21, 2]          # the last token of each sequence
+    assert dec["context_lens"].tolist() == [9, 6, 3]
+    assert dec["block_tables"].tolist() == [[9, 1, 3], [2, 5, -1], [0, -1, -1]]
+    assert dec["max_query_len"] == 1
+    assert get_attention_context(seqs, [1], True, "cpu")["cu_seqlens_q"].tolist() == [0, 6]
+    assert get_attention_context(seqs, [1], False, "cpu")["context_lens"].tolist() == [6]
+    # a decode step is a verify step without draft tokens: same slots of the cache are read
+    for sid in (1, 4, 7):
+        seqs[sid].draft_start_num_tokens = seqs[sid].num_tokens
+    ver = build_verify_context(seqs, [7, 1, 4], device="cpu")
+    assert ver["context_lens"].tolist() == dec["context_lens"].tolist()
+    assert ver["block_tables"].tolist() == dec["block_tables"].tolist()
+    assert ver["verify_query_lens"].tolist() == [1, 1, 1] and ver["slot_mapping"].numel() == 0
 
 
 def test_oracle_store_kvcache_semantics():

@@ -95,11 +95,11 @@ def test_static_scratch_call_under_graph_capture(dev):
         call()                                   # warm-up on the capture stream, outside capture
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated(dev)
+    # (a device allocation or a symbol look-up inside the capture would invalidate it and fail here;
+    # torch's own allocator cannot be used as a witness: beginning a capture allocates its RNG state)
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
         call()
-    assert torch.cuda.memory_allocated(dev) == before, "the captured call allocated device memory"
     for rep in range(4):
         out_f32.fill_(float("nan")); out_act.zero_(); idx.fill_(-1)
         if rep == 2:                             # other inputs through the same graph, then the first ones again
