@@ -32,6 +32,9 @@ HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 HEADLINE = "qwen3_30b_stack48_t256"
 OTHERS = ("mixtral_t160", "mixtral_t5", "qwen3_30b_t64_zipf", "qwen3_235b_t4096")
+# beside the five configurations: the 48-layer stack under a Zipf-skewed router (no CPU baseline: the
+# arithmetic per token is that of the headline)
+SKEWED = ("qwen3_30b_stack48_t256_zipf",)
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
 
 
@@ -265,7 +268,7 @@ def bench_stack(wl, dev, steps, warmup, with_cpu, cpu_layers=4):
 
     k = dict(zip(_lib.KERNEL_NAMES, stage_ms))
     # active experts per layer: re-run the layers' routing through the whole-block outputs
-    active = _stack_active_experts(stack, x, wl)
+    active, max_rows = _stack_active_experts(stack, x, wl)
     dom_kernel, dom_ms, dom_bytes = _dominant(wl, k, sum(active), wl.layers)
     alg_bytes = sum(wl.algorithmic_bytes(a, out_bytes=2) for a in active)
     res = {
@@ -275,6 +278,7 @@ def bench_stack(wl, dev, steps, warmup, with_cpu, cpu_layers=4):
         "ms_per_step_with_kernel_events": round(ms_events, 5),
         "resident_weight_gb": round(wl.layers * wl.E * wl.expert_w4_bytes / 1e9, 3),
         "active_experts_per_layer_mean": round(sum(active) / len(active), 2),
+        "max_rows_per_expert": {"mean_over_layers": round(sum(max_rows) / len(max_rows), 1), "max": max(max_rows)},
         "layer_hbm_frac": round(alg_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
         "kernel_ms": {n: round(v, 5) for n, v in k.items()},
         "kernel_ms_sum": round(sum(stage_ms), 5),
@@ -369,20 +373,22 @@ def bench_attention(dev, steps, warmup, with_cpu):
 
 
 def _stack_active_experts(stack, x, wl):
-    """Experts with at least one token, per layer, from the counts the whole-block call returns."""
+    """Experts with at least one token and the largest per-expert row count, per layer, from the
+    counts the whole-block call returns."""
     import torch
     from on_device_sd_amd import ops
     plan = ops.MoeForwardPlan(wl.T, wl.H, wl.E, wl.K, wl.I, wl.renorm, wl.act_dtype, x.device,
                               want_f32=False, want_act=True)
     h = x.clone()
-    active = []
+    active, max_rows = [], []
     for l in range(stack.L):
         o = plan.run(h, stack.gate[l], stack.tables[l], stack.norm[l], stack.config.rms_norm_eps,
                      add_residual=True)
         active.append(int((o.counts > 0).sum()))
+        max_rows.append(int(o.counts.max()))
         h = o.out_act.clone()
     torch.cuda.synchronize()
-    return active
+    return active, max_rows
 
 
 def _time_cpu(run, budget_s, min_runs=2, max_runs=10):
@@ -503,6 +509,7 @@ def main():
     if args.workload is None:
         line["workloads"] = [run_workload(CONFIGS[name], dev, args.steps, args.warmup, not args.no_cpu)
                              for name in OTHERS]
+        line["workloads"] += [run_workload(CONFIGS[name], dev, args.steps, args.warmup, False) for name in SKEWED]
         line["workloads"].append(bench_attention(dev, args.steps, args.warmup, not args.no_cpu))
     print(json.dumps(line))
 

@@ -586,7 +586,7 @@ struct ExpertsPlan {
 
 // one-launch expert kernel (experts_fused.hip)
 void odsd_launch_experts_fused(FusedParams &fp, int E, hipStream_t st);
-int odsd_fused_supported(int H, int I, int S);
+int odsd_fused_supported(int H, int I, int S, int E);
 int odsd_fused_dispatch_supported(int P);
 
 // Choices are functions of the shape only (the per-expert counts live on the device).
@@ -669,7 +669,7 @@ static ExpertsPlan experts_plan(const odsd_moe_shape *s) {
     p.S = 1;
     if (s->T > 16 && mean_rows >= 8 && mean_rows <= 20 && (s->max_rows <= 0 || s->max_rows <= ODSD_ONE_LAUNCH_ROWS)) {
         int S = 256 / s->E;
-        if (S >= 1 && S <= 2 && s->E * S >= 192 && odsd_fused_supported(s->H, s->I, S)) {
+        if (S >= 1 && S <= 2 && s->E * S >= 192 && odsd_fused_supported(s->H, s->I, S, s->E)) {
             p.fused = 1;
             p.S = S;
             const size_t need = odsd_round_up((size_t)S * (size_t)P * s->H * sizeof(half_t), 256);

@@ -26,6 +26,14 @@
 // Workgroups hold 157 KB of LDS, so exactly one is resident per CU: E*S is chosen near the CU
 // count and every workgroup streams the same number of bytes.
 //
+// Skewed routing.  A pass holds 16*MB rows.  The rows of an expert beyond its first pass form further
+// units of work (expert, slice, pass), and these are NOT left to the expert's own two workgroups
+// (which would stream their slices again and again while the rest of the chip has finished): every
+// workgroup knows the row count of every expert, so all of them derive the same list of overflow
+// units and the same order of helpers -- the workgroups with the fewest rows of their own first --
+// and helper r takes units r, r + grid, ...  No queue, no atomics, no waiting between workgroups;
+// with no expert beyond one pass (the usual case) nothing of this runs.
+//
 // Replaces the same reference code as the streaming kernels: the three F.linear calls of
 // expert_forward_with_weights (demo/src/layers/mlp.py:227-230) inside the per-expert loop of
 // demo/src/model/qwen3_runner.py:303-380.
@@ -59,6 +67,11 @@ __device__ __forceinline__ half8_t raw_word(const RawConsts &c, const uint32_t x
 #define ODSD_RAW_OFFSET_HI 64.0f
 
 typedef float float2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint64_t uniform_u64(const uint64_t v) {
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return ((uint64_t)hi << 32) | lo;
+}
 
 // Nothing moves across this point: the scheduling fence binds the machine scheduler, the empty
 // statement with a memory clobber binds the instruction selector's ordering of a long straight-line
@@ -102,81 +115,174 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
     __shared__ float2_t cx[(G_UP + GS) * MB * 16];
     __shared__ int32_t rows_lds[16 * MB];        // DISP: tokens of the pass's rows
     __shared__ int32_t wsum[2][WAVES];           // DISP: per-wavefront totals (pairs of e, pairs below e)
+    __shared__ int32_t cnt_all[ODSD_FUSED_MAX_E];   // DISP: rows of every expert (histogram of the id list)
+    __shared__ int32_t helper_lds[WAVES];        // overflow units: per-wavefront counts of the helper order
 
-    const int b = blockIdx.x;
-    const int e = b / p.S, s = b - e * p.S;
-    // everything the prologue depends on is requested at once (one round trip, not three)
-    const uint64_t *trow = p.table + (size_t)e * ODSD_TABLE_COLS;
-    const uint64_t t_gu_q = trow[0], t_gu_sz = trow[1], t_dn_q = trow[2], t_dn_sz = trow[3];
-    int M_e, base;
+    constexpr int ROWS = 16 * MB;                // rows of one pass
     constexpr int NID = DISP ? 4 * DISP : 1;     // ids per thread
-    int rk[NID];                                 // DISP: rank of this thread's pairs inside the expert, or -1
-#pragma unroll
-    for (int j = 0; j < NID; ++j) rk[j] = -1;
-    int pair0 = 0;
-    if (DISP) {
-        const int tid_ = threadIdx.x, lane_ = tid_ & 63, wave_ = tid_ >> 6;
-        pair0 = NID * tid_;
-        int id[NID];
+    const int b = blockIdx.x;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, kq = lane >> 4;
+    const int pair0 = NID * tid;
+
+    // The expert ids of this thread's pairs (DISP): 4 or 8 consecutive ones, one or two 16-byte loads.
+    auto load_ids = [&](int (&id)[NID]) {
 #pragma unroll
         for (int v = 0; v < NID / 4; ++v) {
             uint4_t w = {~0u, ~0u, ~0u, ~0u};
             if (pair0 + 4 * v < p.P) w = *(const uint4_t *)(p.idx + pair0 + 4 * v);   // P is a multiple of 4
             id[4 * v] = (int)w.x; id[4 * v + 1] = (int)w.y; id[4 * v + 2] = (int)w.z; id[4 * v + 3] = (int)w.w;
         }
+    };
+    // DISP: one scan of the id list for expert e_: its row count, its first slot, and the tokens of its
+    // rows m0_ .. m0_ + ROWS - 1 (into rows_lds); the order of the pair list is kept (stable).  `first`
+    // (the workgroup's own unit): the histogram of all experts is made on the way, and slice 0 writes
+    // counts[e], offsets[e] and the slots of the expert's pairs -- what a separate dispatch kernel and
+    // two dependent loads per workgroup did before.  Ends with a barrier.
+    auto scan_for = [&](const int (&id)[NID], const int e_, const int m0_, const bool first, const bool writer,
+                        int &M_out, int &base_out) {
         int cm = 0, cl = 0;
 #pragma unroll
         for (int j = 0; j < NID; ++j) {
-            cm += id[j] == e;
-            cl += (uint32_t)id[j] < (uint32_t)e; // ids outside [0, E) belong to nobody
+            cm += id[j] == e_;
+            cl += (uint32_t)id[j] < (uint32_t)e_;   // ids outside [0, E) belong to nobody
+        }
+        if (first) {
+#pragma unroll
+            for (int j = 0; j < NID; ++j)
+                if ((uint32_t)id[j] < (uint32_t)p.E) atomicAdd(&cnt_all[id[j]], 1);
         }
         // counts of at most NID per lane: one ballot per bit gives the prefix over the lower lanes and the total
         constexpr int NBITS = DISP == 1 ? 3 : 4;
         int pre = 0, tot_eq = 0, tot_lt = 0;
 #pragma unroll
-        for (int b = 0; b < NBITS; ++b) {
-            const uint64_t mb = __ballot(cm & (1 << b)), lb = __ballot(cl & (1 << b));
-            pre += mask_rank(mb) << b;
-            tot_eq += __popcll(mb) << b;
-            tot_lt += __popcll(lb) << b;
+        for (int bit = 0; bit < NBITS; ++bit) {
+            const uint64_t mb = __ballot(cm & (1 << bit)), lb = __ballot(cl & (1 << bit));
+            pre += mask_rank(mb) << bit;
+            tot_eq += __popcll(mb) << bit;
+            tot_lt += __popcll(lb) << bit;
         }
-        if (lane_ == 0) {
-            wsum[0][wave_] = tot_eq;
-            wsum[1][wave_] = tot_lt;
+        if (!first) __syncthreads();              // the previous unit is done with wsum and rows_lds
+        if (lane == 0) {
+            wsum[0][wave] = tot_eq;
+            wsum[1][wave] = tot_lt;
         }
         __syncthreads();
         int before = 0, tot_m = 0, tot_l = 0;
 #pragma unroll
         for (int w = 0; w < WAVES; ++w) {
             const int a = wsum[0][w];
-            if (w < wave_) before += a;
+            if (w < wave) before += a;
             tot_m += a;
             tot_l += wsum[1][w];
         }
-        M_e = tot_m;
-        base = tot_l;
+        M_out = __builtin_amdgcn_readfirstlane(tot_m);
+        base_out = __builtin_amdgcn_readfirstlane(tot_l);
         int rank = before + pre;
+        if (writer && tid == 0) {
+            p.out_counts[e_] = tot_m;
+            p.out_offsets[e_] = tot_l;
+            if (e_ == p.E - 1) p.out_offsets[p.E] = tot_l + tot_m;
+        }
 #pragma unroll
         for (int j = 0; j < NID; ++j) {
-            if (id[j] == e) rk[j] = rank++;
-        }
-        if (s == 0) {
-            if (tid_ == 0) {
-                p.out_counts[e] = M_e;
-                p.out_offsets[e] = base;
-                if (e == p.E - 1) p.out_offsets[p.E] = base + M_e;
-            }
-#pragma unroll
-            for (int j = 0; j < NID; ++j) {
+            if (id[j] == e_) {
+                const int rel = rank - m0_;
+                if (rel >= 0 && rel < ROWS) rows_lds[rel] = (pair0 + j) / p.K;
                 // (the ids come from this library's router, so every pair belongs to some expert's workgroup)
-                if (rk[j] >= 0) p.out_perm[pair0 + j] = base + rk[j];
+                if (writer) p.out_perm[pair0 + j] = tot_l + rank;
+                ++rank;
             }
         }
+        __syncthreads();                          // the row list is complete
+    };
+    // rows of expert x as every workgroup sees them
+    auto rows_of = [&](const int x) -> int { return DISP ? cnt_all[x] : p.counts[x]; };
+
+    // ---- the workgroup's own unit: (expert b / S, slice b % S), the expert's first ROWS rows ----------
+    int e = b / p.S, s = b - e * p.S;
+    // everything the prologue depends on is requested at once (one round trip, not three)
+    const uint64_t *trow = p.table + (size_t)e * ODSD_TABLE_COLS;
+    uint64_t t_gu_q = trow[0], t_gu_sz = trow[1], t_dn_q = trow[2], t_dn_sz = trow[3];
+    int M_e, base, m0 = 0;
+    if (DISP) {
+        int id[NID];
+        load_ids(id);                             // on its way together with the table row
+        for (int x = tid; x < p.E; x += 64 * WAVES) cnt_all[x] = 0;
+        __syncthreads();
+        scan_for(id, e, 0, true, s == 0, M_e, base);
     } else {
         M_e = p.counts[e];
         base = p.offsets[e];
     }
-    if (M_e == 0 || t_gu_q == 0) return;
+    // After its own unit: does any expert have more rows than one pass holds?  (every wavefront looks
+    // at all counts)  If so -- rare -- the overflow units: unit u = (expert, pass >= 1, slice), experts
+    // ascending, passes ascending, slices ascending; helper order = workgroups by (rows of their own
+    // expert, workgroup id) ascending; this workgroup, helper number `helper`, takes units helper,
+    // helper + grid, ...
+    int n_units = 0, helper = 0;
+    auto overflow_plan = [&]() -> bool {
+        bool any_over = false;
+        for (int x = lane; x < p.E; x += 64) any_over |= rows_of(x) > ROWS;
+        if (!__any(any_over)) return false;
+        for (int x = 0; x < p.E; ++x) n_units += ((rows_of(x) + ROWS - 1) / ROWS > 1 ? (rows_of(x) + ROWS - 1) / ROWS - 1 : 0) * p.S;
+        const int mine = rows_of(b / p.S);
+        int below = 0;
+        for (int o = tid; o < (int)gridDim.x; o += 64 * WAVES) {
+            const int oc = rows_of(o / p.S);
+            below += (oc < mine || (oc == mine && o < b)) ? 1 : 0;
+        }
+        below = (int)wave_sum((float)below);      // at most 64 * ceil(grid / 512) per wavefront: exact in fp32
+        __syncthreads();                          // (the own unit's readers of helper_lds's neighbours are done)
+        if (lane == 0) helper_lds[wave] = below;
+        __syncthreads();
+        for (int w = 0; w < WAVES; ++w) helper += helper_lds[w];
+        helper = __builtin_amdgcn_readfirstlane(helper);
+        n_units = __builtin_amdgcn_readfirstlane(n_units);
+        return true;
+    };
+
+    for (int it = 0;; ++it) {
+    if (it > 0) {
+        if (it == 1 && !overflow_plan()) break;
+        const int u = helper + (it - 1) * (int)gridDim.x;
+        if (u >= n_units) break;
+        // decode unit u
+        int acc_u = 0, ue = 0, upass = 0, us = 0;
+        for (int x = 0; x < p.E; ++x) {
+            const int np = (rows_of(x) + ROWS - 1) / ROWS;
+            const int nu = (np > 1 ? np - 1 : 0) * p.S;
+            if (u < acc_u + nu) {
+                ue = x;
+                upass = 1 + (u - acc_u) / p.S;
+                us = (u - acc_u) % p.S;
+                break;
+            }
+            acc_u += nu;
+        }
+        // (wavefront-uniform values that came through LDS: back into scalar registers, so that the table
+        // row is a scalar load and the buffer resources are built on the scalar unit)
+        e = __builtin_amdgcn_readfirstlane(ue);
+        s = __builtin_amdgcn_readfirstlane(us);
+        m0 = __builtin_amdgcn_readfirstlane(upass) * ROWS;
+        trow = p.table + (size_t)e * ODSD_TABLE_COLS;
+        t_gu_q = trow[0]; t_gu_sz = trow[1]; t_dn_q = trow[2]; t_dn_sz = trow[3];
+        if (DISP) {
+            int id[NID];
+            load_ids(id);
+            scan_for(id, e, m0, false, false, M_e, base);
+        } else {
+            M_e = p.counts[e];
+            base = p.offsets[e];
+        }
+    }
+    if (M_e <= m0 || t_gu_q == 0) continue;
+    // the table row is the same in every lane: say so (the buffer resources built from it must live in
+    // scalar registers, or every load is wrapped in a loop over the distinct values)
+    t_gu_q = uniform_u64(t_gu_q); t_gu_sz = uniform_u64(t_gu_sz);
+    t_dn_q = uniform_u64(t_dn_q); t_dn_sz = uniform_u64(t_dn_sz);
     const global_char *src_c = (const global_char *)p.x16;
     // the expert's packed matrices and their (scale, zero) pairs as buffer resources (reads past
     // the end return zero)
@@ -190,10 +296,6 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
         (void *)(uintptr_t)t_dn_sz, 0, (p.H / 16) * G_DN * 64, 0x00020000);
 
     const RawConsts rc = raw_consts();
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int r = lane & 15, kq = lane >> 4;
 
     // gate_up duty: block pairs of the slice (the slice owns the fused matrix's blocks
     // s*16*GS .. (s+1)*16*GS - 1).  A pair is 2 * G_UP KiB of contiguous tiles -- [gate block][group],
@@ -228,17 +330,10 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
     const int row_in_blk = 4 * quarter + kq;
     constexpr int N_PIECES = G_UP * MB / 2;                   // copies per wavefront
 
-    for (int m0 = 0; m0 < M_e; m0 += 16 * MB) {
-        const int mcnt = min(M_e - m0, 16 * MB);
-        if (DISP) {
-            // tokens of this pass's rows (readers of the previous pass's list passed several barriers ago)
-#pragma unroll
-            for (int j = 0; j < NID; ++j) {
-                const int rel = rk[j] - m0;
-                if (rk[j] >= 0 && rel >= 0 && rel < 16 * MB) rows_lds[rel] = (pair0 + j) / p.K;
-            }
-        }
-        __syncthreads();                                      // the previous pass is done with both LDS areas
+    {
+        const int mcnt = min(M_e - m0, ROWS);
+        // the previous unit is done with both LDS areas (DISP: its scan has passed barriers since)
+        if (!DISP && it > 0) __syncthreads();
         // The pass is compiled once per number of token blocks that hold rows: with a run-time count
         // the values that exist on one path only (fragments, group sums, the second block's partial
         // sums) stay live across the whole unrolled stream.
@@ -453,6 +548,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
         if (MB == 1 || mcnt <= 16) run_pass(std::integral_constant<int, 1>{});
         else run_pass(std::integral_constant<int, MB>{});
     }
+    }   // units
 }
 
 // Shapes the fused kernel is built for; the caller has checked them with odsd_fused_supported().
@@ -472,8 +568,8 @@ int odsd_fused_dispatch_supported(int P) { return P % 4 == 0 && P <= 8 * 512; }
 
 // H = 2048 (4 sub-passes of 8 wavefronts x 4 blocks), slices of 384 features, token rows of one
 // pass within the 128 KB row area
-int odsd_fused_supported(int H, int I, int S) {
-    if (S < 1 || I % (ODSD_GROUP * S)) return 0;
+int odsd_fused_supported(int H, int I, int S, int E) {
+    if (S < 1 || I % (ODSD_GROUP * S) || E > ODSD_FUSED_MAX_E) return 0;
     if (I / (ODSD_GROUP * S) != 3 || I / ODSD_GROUP != 6) return 0;
     if (H != 2048) return 0;
     if ((H / ODSD_GROUP) * 2 > ODSD_FUSED_X_BLOCKS) return 0;

@@ -39,6 +39,7 @@ struct GemmParams {
 
 // Launch parameters of the one-launch expert kernel (experts_fused.hip)
 #define ODSD_FUSED_X_BLOCKS 32   // (group, token block) areas of 4 KiB in its token-row LDS area
+#define ODSD_FUSED_MAX_E 256     // experts it keeps row counts of (one workgroup per expert slice: E * S ~ 256)
 struct FusedParams {
     const uint64_t *table;   // [E][4]
     const half_t *x16;       // activations, fp16 [T][H]

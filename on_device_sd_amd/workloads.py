@@ -61,6 +61,11 @@ CONFIGS = {
                                       renorm=True, act_dtype=torch.bfloat16, zipf_s=1.1),
     "qwen3_30b_stack48_t256": MoEWorkload("qwen3_30b_stack48_t256", T=256, H=2048, E=128, K=8,
                                           I=768, renorm=True, act_dtype=torch.bfloat16, layers=48),
+    # not one of the five configurations: the stack with the router bias of the T = 64 layer, for what
+    # load imbalance does to the whole-block path (hot experts hold up to T rows, many hold two or three)
+    "qwen3_30b_stack48_t256_zipf": MoEWorkload("qwen3_30b_stack48_t256_zipf", T=256, H=2048, E=128, K=8,
+                                               I=768, renorm=True, act_dtype=torch.bfloat16, layers=48,
+                                               zipf_s=1.1),
     "qwen3_235b_t4096": MoEWorkload("qwen3_235b_t4096", T=4096, H=4096, E=128, K=8, I=1536,
                                     renorm=True, act_dtype=torch.bfloat16, regime="prefill"),
 }

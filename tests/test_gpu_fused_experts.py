@@ -136,6 +136,51 @@ def test_whole_block_dispatches_inside_the_expert_kernel(dev, layer, T):
     assert torch.equal(out2.out_f32, out.out_f32) and torch.equal(out2.perm, out.perm)
 
 
+@pytest.mark.parametrize("T,absent", [(256, ()), (160, ()), (256, "hot")])
+def test_whole_block_under_a_skewed_router(dev, layer, T, absent):
+    """A router whose popularity follows Zipf(1.1) (the bias of the T = 64 benchmark layer) at the
+    one-launch kernel's shape: the hot experts hold up to T rows -- several passes of 32 -- and many
+    experts hold one or two.  The rows beyond an expert's first pass are handed to the workgroups
+    with the least work of their own (no queue, no atomics: every workgroup derives the same list
+    from the row counts); routing must be the oracle's bit for bit, outputs within tolerance, and a
+    second run must give the same bits.  `absent` = "hot": the two most popular experts have no
+    weights (their overflow units exist and must be skipped)."""
+    print("fused experts, skewed router", T, absent, flush=True)
+    import math
+    from on_device_sd_amd import ops
+    bank, experts = layer
+    g = torch.Generator().manual_seed(4000 + T)
+    wg = torch.randn(E, H, generator=g) * 0.02
+    rank = torch.randperm(E, generator=g).to(torch.float32) + 1.0
+    bias = -1.1 * torch.log(rank) * (0.5 * 0.02 * math.sqrt(H))
+    wg = (wg + (bias / 8.0)[:, None] * torch.full((H,), 1.0 / math.sqrt(H))[None, :]).to(torch.bfloat16)
+    x = (torch.randn(T, H, generator=g) + 8.0 / math.sqrt(H)).to(torch.bfloat16)
+    idx, w = orc.route(orc.router_logits(x, wg), K, True)
+    c, o, perm, _ = orc.dispatch(idx, E)
+    assert c.max() > 96 and (c > 32).sum() >= 5, "the case is meant to have several experts beyond one pass"
+    table = bank.table()
+    present = experts
+    if absent == "hot":
+        gone = np.argsort(-c)[:2].tolist()
+        table = table.clone()
+        for e in gone:
+            table[e] = 0
+        present = {e: ex for e, ex in experts.items() if e not in gone}
+    out = ops.moe_forward(x.to(dev), wg.to(dev), table, K, I, renorm=True)
+    torch.cuda.synchronize()
+    assert np.array_equal(out.idx.cpu().numpy(), idx)
+    assert np.array_equal(out.counts.cpu().numpy(), c)
+    assert np.array_equal(out.offsets.cpu().numpy(), o)
+    assert np.array_equal(out.perm.cpu().numpy(), perm)
+    ref = orc.moe_forward(x, idx, w, present)
+    mx, mean = check_output(out.out_f32, ref)
+    check_output_relative(out.out_f32, ref)
+    print(f"  largest expert {c.max()} rows, {int((c > 32).sum())} experts beyond one pass, {int((c == 0).sum())} without rows; "
+          f"vs oracle: max-abs {mx:.3e} mean-abs {mean:.3e}", flush=True)
+    out2 = ops.moe_forward(x.to(dev), wg.to(dev), table, K, I, renorm=True)
+    assert torch.equal(out2.out_f32, out.out_f32) and torch.equal(out2.perm, out.perm)
+
+
 def test_fused_experts_absent_and_substituted_experts(dev, layer):
     """Table rows of the one-launch path: an expert without weights (row of zeros) contributes
     nothing, as the reference skips experts without parameters (qwen3_runner.py:330-333); a row that
