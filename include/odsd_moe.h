@@ -176,9 +176,9 @@ int odsd_experts_w4(const odsd_moe_shape *s, const void *x_f16, const uint64_t *
 /* The three kernels of odsd_experts_w4 one by one (same arguments, same results), for
  * callers that keep h / y themselves or time the stages:
  *   h_f16 fp16 [P, I] in slot order; y: a buffer of odsd_w4_down_splits(s)*P*H*4 bytes that
- *   odsd_w4_down fills and odsd_combine reads -- float [splits][P][H] partial sums over slices
- *   of I, which odsd_combine adds in slice order, or, when the reduction is not split
- *   (splits == 1), fp16 [P][H].
+ *   odsd_w4_down fills and odsd_combine reads -- [splits][P][H] partial sums over slices of I,
+ *   which odsd_combine adds in slice order: fp16 values (a value beyond +-65504 saturates), except
+ *   for calls with T <= 16, which keep float partial sums when the reduction is split.
  * They stand in for the three F.linear calls of mlp.py:227-230 (gate/up fused with
  * SiLU*mul, then down) and the indexed "+=" of qwen3_runner.py:363. */
 int     odsd_w4_gate_up_silu(const odsd_moe_shape *s, const void *x_f16, const uint64_t *table,

@@ -421,7 +421,7 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
                             const int n = (blk0 + i) * 16 + kq * 4;
                             if (p.y_f16) {
                                 const float4_t v = acc[i][m];
-                                *(half4_t *)((half_t *)p.y + slot * p.ldo + n) =
+                                *(half4_t *)((half_t *)p.y + ((size_t)ks * p.P + slot) * p.ldo + n) =
                                     half4_t{f32_to_f16_sat(v.x), f32_to_f16_sat(v.y), f32_to_f16_sat(v.z), f32_to_f16_sat(v.w)};
                             } else {
                                 *(float4_t *)(p.y + ((size_t)ks * p.P + slot) * p.ldo + n) = acc[i][m];
@@ -445,7 +445,8 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
 // and weight first, then KB independent row loads -- and added in k order; with the generic loop
 // every row load waits for the one before it (its address hangs on a branch), which is what the
 // kernel's time consists of at K = 8.
-// YH: 0 = y holds fp32 partial sums of KS slices; 1 = complete sums as fp16; 2 = two fp16 slices
+// YH: 0 = y holds fp32 partial sums of KS slices; 1 = complete sums as fp16; 2 = KS fp16 slices (the
+// batched form, KB > 0, takes exactly two)
 template <typename XT, int YH, bool STATS, int KB>
 __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ y, const int32_t *__restrict__ idx,
                                                       const float *__restrict__ w,
@@ -524,12 +525,14 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
             if (slot < 0 || e < 0 || e >= E || table[(size_t)e * ODSD_TABLE_COLS] == 0) continue;
             float4_t v;
             if (YH) {
-                // fp16 values: complete sums (YH == 1) or the partial sums of two slices (YH == 2)
+                // fp16 values: complete sums (YH == 1) or the partial sums of KS slices (YH == 2)
                 const half4_t hv = *(const half4_t *)((const half_t *)y + (size_t)slot * H + c);
                 v = float4_t{(float)hv.x, (float)hv.y, (float)hv.z, (float)hv.w};
                 if (YH == 2) {
-                    const half4_t hs = *(const half4_t *)((const half_t *)y + ((size_t)P + slot) * H + c);
-                    v += float4_t{(float)hs.x, (float)hs.y, (float)hs.z, (float)hs.w};
+                    for (int sl = 1; sl < KS; ++sl) {      // further slices, in slice order
+                        const half4_t hs = *(const half4_t *)((const half_t *)y + ((size_t)sl * P + slot) * H + c);
+                        v += float4_t{(float)hs.x, (float)hs.y, (float)hs.z, (float)hs.w};
+                    }
                 }
             } else {
                 v = *(const float4_t *)(y + (size_t)slot * H + c);
@@ -648,13 +651,15 @@ static ExpertsPlan experts_plan(const odsd_moe_shape *s) {
     }
     // every split must own at least one group
     while (p.KS > 1 && ((G_dn + p.KS - 1) / p.KS) * (p.KS - 1) >= G_dn) p.KS--;
-    // Without a split of the reduction the down projection's outputs are complete sums: they are
-    // stored as fp16 (3 more bits than the bf16 the reference keeps its expert outputs in), half the
-    // bytes to write and to read back in the combine (at prefill shapes fp32 would be 0.5 GB per
-    // layer each way).  Split reductions leave fp32 partial sums, added in order by the combine.
-    p.y_f16 = p.KS == 1;
+    // The down projection's outputs are stored as fp16 (3 more bits than the bf16 the reference keeps
+    // its expert outputs in): half the bytes to write and to read back in the combine (at prefill
+    // shapes fp32 would be 0.5 GB per layer each way) -- complete sums without a split of the
+    // reduction, one fp16 partial sum per slice with one (added in slice order by the combine; at the
+    // Mixtral T = 160 shape the fp32 form wrote and re-read 21 MB per layer).  Calls with at most 16
+    // tokens keep fp32 partial sums: they split deepest (up to 16 slices) and move next to nothing.
+    p.y_f16 = p.KS == 1 || p.MB >= 2;
     p.h_bytes = odsd_round_up((size_t)(P > 0 ? P : 1) * s->I * sizeof(half_t), 256);
-    p.y_bytes = odsd_round_up((size_t)p.KS * (size_t)(P > 0 ? P : 1) * s->H * sizeof(float), 256);
+    p.y_bytes = odsd_round_up((size_t)p.KS * (size_t)(P > 0 ? P : 1) * s->H * (p.y_f16 ? sizeof(half_t) : sizeof(float)), 256);
     // The one-launch expert kernel serves calls where nearly every expert has rows and a pass holds
     // them all (8 to 20 rows per expert on average, at most 32 per pass; measured against the
     // two-launch plan on uniform routing it wins up to 20 and loses from 24 on, where many experts
@@ -838,13 +843,13 @@ static int launch_combine(const odsd_moe_shape *s, const void *y_, const int32_t
     if (row_ss && !out_act) return ODSD_ERR_NULL;
     if (!odsd_aligned16(y) || (out_f32 && !odsd_aligned16(out_f32))) return ODSD_ERR_ALIGN;
     ExpertsPlan pl = experts_plan(s);
-    if (y_slices > 2) return ODSD_ERR_UNSUPPORTED;          // fp16 partial sums: one or two slices
     if (y_slices > 0) { pl.KS = y_slices; pl.y_f16 = 1; }
     const int P = s->T * s->K;
     const int nchunk = (s->H / 4 + 255) / 256;
     if ((int64_t)nchunk * s->T > 0x7fffffffLL) return ODSD_ERR_UNSUPPORTED;
     const dim3 grid((unsigned)(nchunk * s->T));
-    const bool batched = (pl.KS == 1 || pl.y_f16) && s->K % 4 == 0;      // rows of 4 pairs fetched together (8: no faster)
+    // rows of 4 pairs fetched together (8: no faster): complete sums, or two fp16 slices
+    const bool batched = (pl.KS == 1 || (pl.y_f16 && pl.KS == 2)) && s->K % 4 == 0;
 #define COMBINE_GO(XT, YH, ST)                                                                          \
     do {                                                                                                \
         if (batched)                                                                                    \
@@ -858,7 +863,7 @@ static int launch_combine(const odsd_moe_shape *s, const void *y_, const int32_t
     } while (0)
 #define COMBINE_Y(XT, ST)                                    \
     do {                                                     \
-        if (pl.y_f16 && pl.KS == 2) COMBINE_GO(XT, 2, ST);   \
+        if (pl.y_f16 && pl.KS >= 2) COMBINE_GO(XT, 2, ST);   \
         else if (pl.y_f16) COMBINE_GO(XT, 1, ST);            \
         else COMBINE_GO(XT, 0, ST);                          \
     } while (0)

@@ -309,7 +309,7 @@ __global__ __launch_bounds__(512, 2) void w4_gemm_prefill_kernel(const GemmParam
                             const int n = (cblk0 + i) * 16 + kq * 4;
                             if (p.y_f16) {
                                 const float4_t v = acc[i][m];
-                                *(half4_t *)((half_t *)p.y + slot * p.ldo + n) =
+                                *(half4_t *)((half_t *)p.y + ((size_t)ks * p.P + slot) * p.ldo + n) =
                                     half4_t{f32_to_f16_sat(v.x), f32_to_f16_sat(v.y), f32_to_f16_sat(v.z), f32_to_f16_sat(v.w)};
                             } else {
                                 *(float4_t *)(p.y + ((size_t)ks * p.P + slot) * p.ldo + n) = acc[i][m];

@@ -15,8 +15,8 @@ struct GemmParams {
     const int32_t *counts;
     const int32_t *offsets;
     half_t *h16;             // MODE 0 output [P][I]
-    float *y;                // MODE 1 output [KS][P][ldo] fp32, or [P][ldo] fp16 when y_f16
-    int y_f16;               // unsplit reduction: one fp16 value per output instead of fp32 partials
+    float *y;                // MODE 1 output [KS][P][ldo]: fp32 partial sums, or fp16 ones when y_f16
+    int y_f16;               // the partial (KS == 1: complete) sums are stored as fp16
     int src_ld;              // elements per source row (= reduction length Kd)
     int G;                   // groups of 128 in the reduction dimension
     int NBLK;                // 16-row blocks of the (fused) weight matrix
