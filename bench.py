@@ -270,7 +270,7 @@ def bench_stack(wl, dev, steps, warmup, with_cpu, cpu_layers=4):
     stack.graph = None
 
     # the same K steps once more (eager) with every kernel launch carrying its start / stop events
-    events = [[_hip.EventList(2 * _lib.N_KERNELS) for _ in range(wl.layers)] for _ in range(steps)]
+    events = [_hip.EventList(wl.layers * 2 * _lib.N_KERNELS) for _ in range(steps)]
     masks = [None] * steps
     stack.forward_events(x, events[0])
     torch.cuda.synchronize()
@@ -284,7 +284,7 @@ def bench_stack(wl, dev, steps, warmup, with_cpu, cpu_layers=4):
     for i in range(steps):
         tot = [0.0] * _lib.N_KERNELS
         for l in range(wl.layers):
-            for s, v in enumerate(events[i][l].kernel_ms(masks[i][l])):
+            for s, v in enumerate(events[i].kernel_ms_at(l * 2 * _lib.N_KERNELS, masks[i][l], _lib.N_KERNELS)):
                 tot[s] += v
         per_step.append(tot)
     stage_ms = _stage_stats(per_step)

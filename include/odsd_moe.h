@@ -29,6 +29,8 @@
  *                      ExpertOperator.expert_forward           demo/src/operators/base_operator.py:19-34
  *   odsd_moe_forward   Qwen3MoELayerWithWeights.forward        demo/src/layers/moe_layer.py:193-254
  *                      ModelRunner.forward_moe                 demo/src/core/model_runner.py:175-193
+ *   odsd_moe_stack_forward  Qwen3DecoderLayer.forward (MoE half), layer after layer
+ *                                                              demo/src/layers/decoder_layer.py:126-140
  *   odsd_rmsnorm       RMSNorm.rms_forward                     demo/src/layers/layernorm.py:21-27
  *   odsd_w4_quantize   quantize_tensor (form, per group)       pre_exp/expert_skip_prediction/quant.py:85-108
  *   odsd_w4_pack       (no counterpart: the reference holds fp16/bf16 weights only;
@@ -48,8 +50,9 @@ extern "C" {
 
 /* 110: events / static forms of the whole block, KV store, paged and packed attention added (100: the MoE block)
  * 112: odsd_moe_shape.max_rows (was reserved, 0 keeps the old meaning), odsd_experts_one_launch
- * 113: odsd_moe_static_init */
-#define ODSD_VERSION 113
+ * 113: odsd_moe_static_init
+ * 114: odsd_moe_stack_forward, odsd_moe_stack_forward_events */
+#define ODSD_VERSION 114
 
 typedef enum odsd_status {
     ODSD_OK = 0,
@@ -216,6 +219,22 @@ int odsd_moe_forward(const odsd_moe_shape *s, const void *x, const void *norm_we
                      const double *row_sumsq_in, double *row_sumsq_out,
                      void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---- A stack of blocks ------------------------------------------------------------------------ */
+/* n_layers blocks in a row on one hidden state:  h <- h + MoE_l(RMSNorm_l(h)),  l = 0 .. n_layers-1
+ * (Qwen3DecoderLayer.forward without its attention half, demo/src/layers/decoder_layer.py:126-140,
+ * looped over the layers as the model's forward does), with no host round trip between the blocks.
+ *   x [T,H] act_dtype (not written); out [T,H] act_dtype: the hidden state after the last block
+ *   norm_w, gate_w, tables: HOST arrays of n_layers device pointers -- per layer the RMSNorm weight
+ *   [H], the router weight [E,H] (both act_dtype) and the expert table (as for odsd_moe_forward)
+ * Every layer has the shape *s.  Results are those of n_layers odsd_moe_forward calls with
+ * norm_weight and add_residual set, bit for bit (the same kernels; every block after the first takes
+ * its RMSNorm statistic from the previous block's combine). */
+size_t odsd_moe_stack_workspace_bytes(const odsd_moe_shape *s);
+int    odsd_moe_stack_forward(const odsd_moe_shape *s, int32_t n_layers, const void *x,
+                              const void *const *norm_w, const void *const *gate_w,
+                              const uint64_t *const *tables, float eps, void *out,
+                              void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---- KV-cache store (the attention step next to the block) --------------------------------- */
 /* Rows of this step's keys and values to their slots of the paged cache: for i in [0, N)
  *   row = src_index ? src_index[i] : i;  slot = slot_mapping[i];
@@ -299,6 +318,15 @@ int odsd_moe_forward_events(const odsd_moe_shape *s, const void *x, const void *
                             const double *row_sumsq_in, double *row_sumsq_out,
                             void *workspace, size_t workspace_bytes, void *stream,
                             void *const *events, uint32_t *launched_mask);
+
+/* The stack call with every kernel timed (measurement only, as odsd_moe_forward_events): events =
+ * n_layers * 2 * ODSD_N_KERNELS handles, layer l using events[l * 2 * ODSD_N_KERNELS ..];
+ * launched_masks [n_layers] (host) gets the slots each layer launched. */
+int odsd_moe_stack_forward_events(const odsd_moe_shape *s, int32_t n_layers, const void *x,
+                                  const void *const *norm_w, const void *const *gate_w,
+                                  const uint64_t *const *tables, float eps, void *out,
+                                  void *workspace, size_t workspace_bytes, void *stream,
+                                  void *const *events, uint32_t *launched_masks);
 
 /* odsd_moe_forward without a workspace argument and without any allocation, for callers that
  * cannot call hipMalloc: code under HIP graph capture, tight serving loops, harnesses that

@@ -75,6 +75,11 @@ class EventList:
         slot whose bit is set in ``mask``, 0.0 for the others."""
         return [self.elapsed_ms(2 * k, 2 * k + 1) if (mask >> k) & 1 else 0.0 for k in range(self.n // 2)]
 
+    def kernel_ms_at(self, base: int, mask: int, n_slots: int) -> List[float]:
+        """The same for a list that holds the events of several calls one after the other: the
+        ``n_slots`` kernel slots whose events start at index ``base``."""
+        return [self.elapsed_ms(base + 2 * k, base + 2 * k + 1) if (mask >> k) & 1 else 0.0 for k in range(n_slots)]
+
     def __del__(self):
         try:
             rt = runtime()

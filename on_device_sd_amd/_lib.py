@@ -65,6 +65,10 @@ SIGNATURES = {
     "odsd_varlen_attention_workspace_bytes": (C.c_size_t, [C.c_int32] * 6),
     "odsd_moe_forward_events": (C.c_int, [_SP, _P, _P, C.c_float, _P, _P, C.c_int32, _P, _P, _P, _P, _P,
                                           C.c_size_t, _P, _P, _P]),
+    "odsd_moe_stack_workspace_bytes": (C.c_size_t, [_SP]),
+    "odsd_moe_stack_forward": (C.c_int, [_SP, C.c_int32, _P, _P, _P, _P, C.c_float, _P, _P, C.c_size_t, _P]),
+    "odsd_moe_stack_forward_events": (C.c_int, [_SP, C.c_int32, _P, _P, _P, _P, C.c_float, _P, _P, C.c_size_t, _P,
+                                                _P, _P]),
     "odsd_moe_static_init": (C.c_int, []),
     "odsd_moe_forward_static": (C.c_int, [_SP, _P, _P, C.c_float, _P, _P, C.c_int32, _P, _P, _P, _P, _P,
                                           _P, _P, _P, _P, _P]),

@@ -142,6 +142,107 @@ extern "C" int odsd_moe_forward_events(const odsd_moe_shape *s, const void *x, c
     return rc;
 }
 
+// ---- a stack of blocks ------------------------------------------------------------------------------
+// L layers of  h = h + MoE_l(RMSNorm_l(h))  (Qwen3DecoderLayer.forward without attention,
+// demo/src/layers/decoder_layer.py:126-140, looped over the layers) in one call: the blocks run as
+// odsd_moe_forward would, every block after the first with its RMSNorm folded into the router kernel
+// through the row statistic that the previous block's combine leaves.
+struct StackLayout {
+    size_t moe, hbuf[2], rowss[2], total;
+};
+
+static StackLayout stack_layout(const odsd_moe_shape *s) {
+    StackLayout l;
+    const size_t T = s->T > 0 ? s->T : 1;
+    const size_t act = s->act_dtype == ODSD_DT_F32 ? 4 : 2;
+    size_t o = 0;
+    auto take = [&](size_t bytes) { const size_t at = o; o += odsd_round_up(bytes, 256); return at; };
+    l.moe = take(moe_layout(s).total);
+    l.hbuf[0] = take(T * s->H * act);
+    l.hbuf[1] = take(T * s->H * act);
+    const size_t nchunk = ((size_t)s->H + 1023) / 1024;
+    l.rowss[0] = take(T * nchunk * sizeof(double));
+    l.rowss[1] = take(T * nchunk * sizeof(double));
+    l.total = o;
+    return l;
+}
+
+extern "C" size_t odsd_moe_stack_workspace_bytes(const odsd_moe_shape *s) {
+    if (!s || odsd_moe_workspace_bytes(s) == 0) return 0;
+    return stack_layout(s).total;
+}
+
+static int moe_stack_impl(const odsd_moe_shape *s, int32_t n_layers, const void *x, const void *const *norm_w,
+                          const void *const *gate_w, const uint64_t *const *tables, float eps, void *out,
+                          void *workspace, size_t workspace_bytes, void *stream, void *const *events,
+                          uint32_t *masks) {
+    if (!s) return ODSD_ERR_NULL;
+    if (n_layers < 0) return ODSD_ERR_SHAPE;
+    const size_t need = odsd_moe_stack_workspace_bytes(s);
+    if (need == 0) return ODSD_ERR_SHAPE;
+    if (s->T == 0 || n_layers == 0) return ODSD_OK;
+    if (!x || !norm_w || !gate_w || !tables || !out || !workspace) return ODSD_ERR_NULL;
+    for (int l = 0; l < n_layers; ++l)
+        if (!norm_w[l] || !gate_w[l] || !tables[l]) return ODSD_ERR_NULL;
+    if (x == out) return ODSD_ERR_SHAPE;                       // the first block reads x while it writes out
+    if (!odsd_aligned16(workspace) || !odsd_aligned16(out)) return ODSD_ERR_ALIGN;
+    if (workspace_bytes < need) return ODSD_ERR_WORKSPACE;
+    const StackLayout sl = stack_layout(s);
+    const MoeLayout ml = moe_layout(s);
+    char *ws = (char *)workspace;
+    char *mws = ws + sl.moe;
+    void *hbuf[2] = {ws + sl.hbuf[0], ws + sl.hbuf[1]};
+    double *rowss[2] = {(double *)(ws + sl.rowss[0]), (double *)(ws + sl.rowss[1])};
+    OdsdProf prof{nullptr, 0u};
+    auto begin_layer = [&](int l) {
+        if (events) {
+            prof.events = events + (size_t)l * 2 * ODSD_N_KERNELS;
+            prof.launched = 0u;
+            odsd_prof = &prof;
+        }
+    };
+    auto end_layer = [&](int l) {
+        if (events) {
+            masks[l] = prof.launched;
+            odsd_prof = nullptr;
+        }
+    };
+    auto in_of = [&](int l) -> const void * { return l == 0 ? x : hbuf[(l - 1) & 1]; };
+    auto out_of = [&](int l) -> void * { return l == n_layers - 1 ? out : hbuf[l & 1]; };
+
+    for (int l = 0; l < n_layers; ++l) {
+        begin_layer(l);
+        const int rc = moe_forward_impl(s, in_of(l), norm_w[l], eps, gate_w[l], tables[l], 1, nullptr, out_of(l),
+                                        nullptr, nullptr, nullptr, nullptr, nullptr, l > 0 ? rowss[(l - 1) & 1] : nullptr,
+                                        l + 1 < n_layers ? rowss[l & 1] : nullptr, mws, ml.total, stream);
+        end_layer(l);
+        if (rc != ODSD_OK) return rc;
+    }
+    return ODSD_OK;
+}
+
+extern "C" int odsd_moe_stack_forward(const odsd_moe_shape *s, int32_t n_layers, const void *x,
+                                      const void *const *norm_w, const void *const *gate_w,
+                                      const uint64_t *const *tables, float eps, void *out, void *workspace,
+                                      size_t workspace_bytes, void *stream) {
+    return moe_stack_impl(s, n_layers, x, norm_w, gate_w, tables, eps, out, workspace, workspace_bytes, stream,
+                          nullptr, nullptr);
+}
+
+extern "C" int odsd_moe_stack_forward_events(const odsd_moe_shape *s, int32_t n_layers, const void *x,
+                                             const void *const *norm_w, const void *const *gate_w,
+                                             const uint64_t *const *tables, float eps, void *out, void *workspace,
+                                             size_t workspace_bytes, void *stream, void *const *events,
+                                             uint32_t *launched_masks) {
+    if (!events || !launched_masks) return ODSD_ERR_NULL;
+    for (size_t i = 0; i < (size_t)(n_layers > 0 ? n_layers : 0) * 2 * ODSD_N_KERNELS; ++i)
+        if (!events[i]) return ODSD_ERR_NULL;
+    const int rc = moe_stack_impl(s, n_layers, x, norm_w, gate_w, tables, eps, out, workspace, workspace_bytes, stream,
+                                  events, launched_masks);
+    odsd_prof = nullptr;
+    return rc;
+}
+
 // ---- the whole block for callers that cannot allocate -------------------------------------------
 // The workspace of odsd_moe_forward lives in a device array of this library instead of coming from
 // the caller.  Each GPU holds its own copy of the array at its own address; the address is looked

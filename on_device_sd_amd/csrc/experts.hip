@@ -672,13 +672,16 @@ static ExpertsPlan experts_plan(const odsd_moe_shape *s) {
     // the plan then takes the one-launch kernel only when one pass covers every expert.
     p.fused = 0;
     p.S = 1;
-    if (s->T > 16 && mean_rows >= 8 && mean_rows <= 20 && (s->max_rows <= 0 || s->max_rows <= ODSD_ONE_LAUNCH_ROWS)) {
+    if (s->T > 16 && mean_rows >= 8 && mean_rows <= 20) {
         int S = 256 / s->E;
         if (S >= 1 && S <= 2 && s->E * S >= 192 && odsd_fused_supported(s->H, s->I, S, s->E)) {
-            p.fused = 1;
-            p.S = S;
+            // (the buffer serves either plan: its size does not depend on the caller's statement)
             const size_t need = odsd_round_up((size_t)S * (size_t)P * s->H * sizeof(half_t), 256);
             if (need > p.y_bytes) p.y_bytes = need;
+            if (s->max_rows <= 0 || s->max_rows <= ODSD_ONE_LAUNCH_ROWS) {
+                p.fused = 1;
+                p.S = S;
+            }
         }
     }
     return p;

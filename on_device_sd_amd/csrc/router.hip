@@ -15,6 +15,7 @@
 // Replaces: Qwen3MoEGate.forward (demo/src/layers/moe_layer.py:41-58), the stateless form
 // (:210-216) and GPUOperators.router (demo/src/operators/gpu_operators.py:48-69).
 #include "common.h"
+#include "router_topk.h"
 
 #define ROUTER_MAX_NE 4    // expert tiles (of 16) per wavefront
 #define ROUTER_MAX_V 8     // most logits per lane in the top-k kernel -> E <= 512
@@ -206,13 +207,6 @@ __global__ __launch_bounds__(256) void router_partial_kernel(const XT *__restric
     }
 }
 
-// total order on doubles as unsigned keys: larger value <=> larger key
-__device__ __forceinline__ uint64_t order_key(double v) {
-    if (v == 0.0) v = 0.0;   // -0 and +0 compare equal, so they must share a key
-    const uint64_t b = (uint64_t)__double_as_longlong(v);
-    return (b >> 63) ? ~b : (b | 0x8000000000000000ull);
-}
-
 // V = logits per lane (experts lane, lane + 64, ...): 1, 2, 4 or 8 for E <= 64, 128, 256, 512
 template <int V>
 __global__ __launch_bounds__(256) void router_topk_kernel(const double *__restrict__ partial, int T, int E,
@@ -270,27 +264,7 @@ __global__ __launch_bounds__(256) void router_topk_kernel(const double *__restri
                 }
             }
         }
-        // wavefront arg-max on (key, -expert) with DPP moves; the winner ends up in lane 63
-        uint32_t klo = (uint32_t)bk, khi = (uint32_t)(bk >> 32);
-#define ROUTER_DPP_STEP(CTRL, ROWMASK)                                                              \
-    {                                                                                               \
-        const uint32_t olo = (uint32_t)__builtin_amdgcn_update_dpp((int)klo, (int)klo, CTRL, ROWMASK, 0xF, false); \
-        const uint32_t ohi = (uint32_t)__builtin_amdgcn_update_dpp((int)khi, (int)khi, CTRL, ROWMASK, 0xF, false); \
-        const int oe = __builtin_amdgcn_update_dpp(be, be, CTRL, ROWMASK, 0xF, false);              \
-        const uint64_t ok = ((uint64_t)ohi << 32) | olo, mk = ((uint64_t)khi << 32) | klo;          \
-        const bool better = ok > mk || (ok == mk && oe < be);                                       \
-        klo = better ? olo : klo;                                                                   \
-        khi = better ? ohi : khi;                                                                   \
-        be = better ? oe : be;                                                                      \
-    }
-        ROUTER_DPP_STEP(0x111, 0xF)   // row_shr:1
-        ROUTER_DPP_STEP(0x112, 0xF)   // row_shr:2
-        ROUTER_DPP_STEP(0x114, 0xF)   // row_shr:4
-        ROUTER_DPP_STEP(0x118, 0xF)   // row_shr:8   -> lane 15 of every row holds the row's best
-        ROUTER_DPP_STEP(0x142, 0xA)   // row_bcast:15 into rows 1 and 3
-        ROUTER_DPP_STEP(0x143, 0xC)   // row_bcast:31 into rows 2 and 3 -> lane 63 holds the best
-#undef ROUTER_DPP_STEP
-        const int we = __builtin_amdgcn_readlane(be, 63);   // the same in every lane
+        const int we = wave_argmax(bk, be);   // the same in every lane
         // the winner's logit sits in lane (we & 63), slot (we >> 6)
         double cand = lg[0];
 #pragma unroll

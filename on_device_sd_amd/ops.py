@@ -376,6 +376,45 @@ class MoeForwardPlan:
         return mask.value
 
 
+class MoeStackPlan:
+    """L blocks in a row on one hidden state, h <- h + MoE_l(RMSNorm_l(h)), as ONE library call
+    (``odsd_moe_stack_forward``): pre-sized workspace, the per-layer device pointers as host arrays."""
+
+    def __init__(self, T: int, H: int, E: int, K: int, I: int, renorm: bool, dtype: torch.dtype, device,
+                 norm_weights, gate_weights, tables, eps: float = 1e-6):
+        lib = _lib.load()
+        self.shape = make_shape(T, H, E, K, I, renorm, dtype)
+        nbytes = lib.odsd_moe_stack_workspace_bytes(C.byref(self.shape))
+        if nbytes == 0:
+            raise _lib.OdsdError(f"moe_stack_forward: unsupported shape T={T} H={H} E={E} K={K} I={I}")
+        self.ws = _workspace(nbytes, device)
+        self.L = len(tables)
+        self.eps = eps
+        self._keep = (list(norm_weights), list(gate_weights), list(tables))     # the arrays hold raw addresses
+        arr = lambda ts: (C.c_void_p * self.L)(*[t.data_ptr() for t in ts])
+        self._norm, self._gate, self._tables = arr(norm_weights), arr(gate_weights), arr(tables)
+        self.out = torch.empty(T, H, dtype=dtype, device=device)
+
+    def run(self, x: torch.Tensor) -> torch.Tensor:
+        lib = _lib.load()
+        _lib.check(lib.odsd_moe_stack_forward(C.byref(self.shape), self.L, x.data_ptr(), self._norm, self._gate,
+                                              self._tables, self.eps, self.out.data_ptr(), self.ws.data_ptr(),
+                                              self.ws.numel(), _stream()), "odsd_moe_stack_forward")
+        return self.out
+
+    def run_events(self, events, x: torch.Tensor):
+        """``run`` with every kernel launch timed: ``events`` is an ``_hip.EventList`` of
+        ``L * 2 * _lib.N_KERNELS`` events (layer l: events 2 N l .. 2 N (l+1) - 1).  Returns the list of
+        launched-slot masks, one per layer."""
+        lib = _lib.load()
+        masks = (C.c_uint32 * self.L)()
+        _lib.check(lib.odsd_moe_stack_forward_events(
+            C.byref(self.shape), self.L, x.data_ptr(), self._norm, self._gate, self._tables, self.eps,
+            self.out.data_ptr(), self.ws.data_ptr(), self.ws.numel(), _stream(), events.array, masks),
+            "odsd_moe_stack_forward_events")
+        return list(masks)
+
+
 def moe_forward(x: torch.Tensor, gate_weight: torch.Tensor, table: torch.Tensor, top_k: int,
                 inter: int, renorm: bool, norm_weight: Optional[torch.Tensor] = None,
                 eps: float = 1e-6, add_residual: bool = False, want_f32: bool = True,

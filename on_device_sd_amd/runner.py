@@ -249,9 +249,11 @@ def expert_forward_with_weights(x: torch.Tensor, params: W4ExpertParams,
 
 
 class MoEOnlyStack:
-    """L layers of RMSNorm -> MoE -> residual on a flat [T,H] hidden state, each layer one
-    whole-block call with no host round trip; the hidden state ping-pongs between two
-    buffers.  ``capture()`` records the L calls into a HIP graph for launch-bound shapes."""
+    """L layers of RMSNorm -> MoE -> residual on a flat [T,H] hidden state, with no host round trip.
+    ``forward`` makes one library call for the whole stack (``odsd_moe_stack_forward``: between two
+    blocks the combine, the next RMSNorm and the next router run as one kernel where the shape allows);
+    ``forward_layers`` runs the same layers as L whole-block calls (``odsd_moe_forward``), the hidden
+    state going back and forth between two buffers.  ``capture()`` records ``forward`` into a HIP graph."""
 
     def __init__(self, config: MoEConfig, gate_weights: List[torch.Tensor],
                  norm_weights: List[torch.Tensor], banks: List[W4ExpertBank], T: int):
@@ -268,50 +270,51 @@ class MoEOnlyStack:
                                        config.num_experts_per_token, config.moe_intermediate_size,
                                        config.norm_topk_prob, self.dtype, self.device,
                                        want_f32=False, want_act=False, want_routing=False)
+        self.stack_plan = ops.MoeStackPlan(T, config.hidden_size, config.num_experts,
+                                           config.num_experts_per_token, config.moe_intermediate_size,
+                                           config.norm_topk_prob, self.dtype, self.device, self.norm, self.gate,
+                                           self.tables, config.rms_norm_eps)
         self.buf = [torch.empty(T, config.hidden_size, dtype=self.dtype, device=self.device)
                     for _ in range(2)]
-        # per-row sum of squares of each hidden-state buffer: every layer's combine leaves it for
-        # the next layer, whose RMSNorm is then folded into its router kernel (layer 0 runs the
-        # stand-alone RMSNorm kernel)
+        self.x_in = torch.empty(T, config.hidden_size, dtype=self.dtype, device=self.device)
+        # per-row sum of squares of each hidden-state buffer (layer-by-layer form): every layer's
+        # combine leaves it for the next layer, whose RMSNorm is then folded into its router kernel
+        # (layer 0 runs the stand-alone RMSNorm kernel)
         self.rowss = [ops.row_stats(T, config.hidden_size, self.device) for _ in range(2)]
         self.graph = None
 
-    def _run_layers(self, events=None):
-        masks = []
+    def forward_layers(self, hidden: torch.Tensor) -> torch.Tensor:
+        """The stack as L whole-block calls (eager)."""
+        self.buf[0].copy_(hidden)
         for l in range(self.L):
-            kw = dict(add_residual=True, out_act=self.buf[(l + 1) & 1],
-                      row_sumsq_in=self.rowss[l & 1] if l > 0 else None,
-                      row_sumsq_out=self.rowss[(l + 1) & 1] if l + 1 < self.L else None)
-            if events is None:
-                self.plan.run(self.buf[l & 1], self.gate[l], self.tables[l], self.norm[l],
-                              self.config.rms_norm_eps, **kw)
-            else:
-                masks.append(self.plan.run_events(events[l], self.buf[l & 1], self.gate[l], self.tables[l],
-                                                  self.norm[l], self.config.rms_norm_eps, **kw))
-        return masks
+            self.plan.run(self.buf[l & 1], self.gate[l], self.tables[l], self.norm[l],
+                          self.config.rms_norm_eps, add_residual=True, out_act=self.buf[(l + 1) & 1],
+                          row_sumsq_in=self.rowss[l & 1] if l > 0 else None,
+                          row_sumsq_out=self.rowss[(l + 1) & 1] if l + 1 < self.L else None)
+        return self.buf[self.L & 1]
 
     def forward_events(self, hidden: torch.Tensor, events):
-        """``forward`` (eager) with the kernels of layer l timed by the events ``events[l]``
-        (see ``MoeForwardPlan.run_events``); returns the launched-slot mask of every layer."""
-        self.buf[0].copy_(hidden)
-        return self._run_layers(events)
+        """``forward`` (eager) with every kernel launch timed by ``events`` (see
+        ``MoeStackPlan.run_events``); returns the launched-slot mask of every layer."""
+        self.x_in.copy_(hidden)
+        return self.stack_plan.run_events(events, self.x_in)
 
     def capture(self):
-        """Record the stack into a HIP graph (all kernels, no memset nodes)."""
+        """Record the stack call into a HIP graph (all kernels, no memset nodes)."""
         s = torch.cuda.Stream()
         s.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(s):
-            self._run_layers()   # warm-up outside capture
+            self.stack_plan.run(self.x_in)   # warm-up outside capture
         torch.cuda.current_stream().wait_stream(s)
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
-            self._run_layers()
+            self.stack_plan.run(self.x_in)
         self.graph = g
 
     def forward(self, hidden: torch.Tensor) -> torch.Tensor:
-        self.buf[0].copy_(hidden)
+        self.x_in.copy_(hidden)
         if self.graph is not None:
             self.graph.replay()
         else:
-            self._run_layers()
-        return self.buf[self.L & 1]
+            self.stack_plan.run(self.x_in)
+        return self.stack_plan.out
