@@ -472,15 +472,20 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
                 int slot[KB > 0 ? KB : 1];
                 float wk[KB > 0 ? KB : 1];
                 bool ok[KB > 0 ? KB : 1];
+                uint64_t tq[KB > 0 ? KB : 1];      // first table entry of the pair's expert: 0 = no weights
 #pragma unroll
                 for (int u = 0; u < KB; ++u) {
                     const int pr = t * K + k0 + u;
                     const int sl = perm[pr];
                     const int e = idx[pr];
                     wk[u] = w[pr];
+                    // (the row's address must not wait for the table entry: that would be a third
+                    // dependent round trip to memory -- slot, then table, then row -- in a kernel that
+                    // consists of little else; a pair in range always has a row that exists)
                     const bool in_range = sl >= 0 && e >= 0 && e < E;
-                    ok[u] = in_range && table[(size_t)(in_range ? e : 0) * ODSD_TABLE_COLS] != 0;
-                    slot[u] = ok[u] ? sl : 0;      // a row that exists; its values are discarded below
+                    tq[u] = table[(size_t)(in_range ? e : 0) * ODSD_TABLE_COLS];
+                    ok[u] = in_range;
+                    slot[u] = in_range ? sl : 0;   // a row that exists; its values are discarded below
                 }
                 float4_t v[KB > 0 ? KB : 1];
                 if (YH == 2) {
@@ -509,7 +514,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
                 }
 #pragma unroll
                 for (int u = 0; u < KB; ++u) {
-                    if (ok[u]) {
+                    if (ok[u] && tq[u] != 0) {
                         acc.x = fmaf(wk[u], v[u].x, acc.x);
                         acc.y = fmaf(wk[u], v[u].y, acc.y);
                         acc.z = fmaf(wk[u], v[u].z, acc.z);
