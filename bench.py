@@ -226,6 +226,20 @@ def bench_layer(wl, dev, steps, warmup, with_cpu):
         "kernel_ms_sum": round(sum(stage_ms), 5),
         "roofline": _roofline(wl, dom_ms, dom_bytes, dom_kernel),
     }
+    if k.get("down", 0.0) > 0.0:
+        # the down projection's own stream (a third of an expert's packed bytes) against HBM, or its
+        # flops against the matrix cores at the prefill shape
+        down_bytes = active * (wl.expert_w4_bytes // 3)
+        if wl.regime == "prefill":
+            ach = 2 * wl.pairs * wl.H * wl.I / (k["down"] * 1e-3) / 1e12
+            res["down_roofline"] = {"bound": "mfma", "kernel": "w4_gemm_prefill_kernel<down>", "achieved": round(ach, 2),
+                                    "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                    "frac": round(ach / MFMA_F16_PEAK_TFLOPS, 4), "kernel_ms": round(k["down"], 5)}
+        else:
+            ach = down_bytes / (k["down"] * 1e-3) / 1e9
+            res["down_roofline"] = {"bound": "hbm", "kernel": "w4_gemm_kernel<down>", "achieved": round(ach, 1),
+                                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4),
+                                    "algorithmic_bytes": int(down_bytes), "kernel_ms": round(k["down"], 5)}
     del runner, placements, plan, banks, tables
     if with_cpu:
         res["cpu_baseline"] = cpu_baseline_layer(wl, gate, x, canon)

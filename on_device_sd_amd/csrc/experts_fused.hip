@@ -95,6 +95,20 @@ __device__ __forceinline__ uint64_t uniform_u64(const uint64_t v) {
 //       popcount, the order of the pair list is kept: stable), keeps its expert's token rows in LDS
 //       and, as slice 0, writes counts[e], offsets[e] and the slots of its pairs -- what the
 //       separate dispatch kernel and two dependent loads per workgroup did before
+// Timing-only build (-DODSD_TIMELINE, `make timeline`): every wavefront stamps the 100 MHz real-time
+// counter at eight points and leaves the stamps in a buffer the caller registered, 8 values per
+// (workgroup, wavefront).  The product build compiles none of it.
+#ifdef ODSD_TIMELINE
+__device__ unsigned long long *odsd_tl_buf;
+extern "C" int odsd_debug_timeline(void *buf) {
+    unsigned long long *b = (unsigned long long *)buf;
+    return (int)hipMemcpyToSymbol(HIP_SYMBOL(odsd_tl_buf), &b, sizeof(b));
+}
+#define ODSD_TL(k) tl[k] = __builtin_amdgcn_s_memrealtime()
+#else
+#define ODSD_TL(k)
+#endif
+
 template <int MB, int GS, int WAVES, int G_UP, int G_DN, int DISP>
 __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(const FusedParams p) {
     static_assert(WAVES % 4 == 0 && (8 * GS) % WAVES == 0, "whole gate/up block pairs per wavefront");
@@ -119,6 +133,10 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
     __shared__ int32_t helper_lds[WAVES];        // overflow units: per-wavefront counts of the helper order
 
     constexpr int ROWS = 16 * MB;                // rows of one pass
+#ifdef ODSD_TIMELINE
+    unsigned long long tl[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#endif
+    ODSD_TL(0);
     constexpr int NID = DISP ? 4 * DISP : 1;     // ids per thread
     const int b = blockIdx.x;
     const int tid = threadIdx.x;
@@ -244,6 +262,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
         return true;
     };
 
+    ODSD_TL(1);                                  // own id scan done
     for (int it = 0;; ++it) {
     if (it > 0) {
         if (it == 1 && !overflow_plan()) break;
@@ -381,6 +400,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
         for (int d = 0; d < DEPTH; ++d) load_u(d, d);
         ODSD_WAIT_VMCNT(4 * DEPTH);                           // the copies have landed; 4 loads per ring step are younger
         __builtin_amdgcn_s_barrier();
+        ODSD_TL(2);                                           // token rows in LDS
 
         // Sums of one (group, token block): the lane reads its four B fragments (token row r, columns
         // 32 j + 8 kq ..), adds the values at the 1024-offset positions and at the 64-offset positions
@@ -407,6 +427,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
             if (bi % MB < nmb) group_sums(xs_raw + bi * XBLK, cx + bi * 16);
         }
         __syncthreads();
+        ODSD_TL(3);                                           // group sums of the token rows
 
         // One step = one group of one block pair: B fragments of the group from LDS, the slot's two
         // tiles expanded to fp16, the slot refilled with the step DEPTH ahead, 2 x MB x 4 MFMAs.
@@ -509,11 +530,14 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
                 }
             }
         }
+        ODSD_TL(4);                                           // this wavefront's gate_up stream done
         __syncthreads();                                      // h is complete
+        ODSD_TL(5);
         for (int bi = wave; bi < GS * MB; bi += WAVES) {
             if (bi % MB < nmb) group_sums(hs_raw + bi * XBLK, cx + (G_UP * MB + bi) * 16);
         }
         __syncthreads();
+        ODSD_TL(6);                                           // group sums of h
 
         // down: step u = group u % GS of output block pair u / GS, against h from LDS; the slice's
         // partial sums are stored as fp16 when a pair's last group is done
@@ -549,6 +573,13 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void w4_expert_fused_kernel(
         else run_pass(std::integral_constant<int, MB>{});
     }
     }   // units
+#ifdef ODSD_TIMELINE
+    ODSD_TL(7);
+    if (odsd_tl_buf && (threadIdx.x & 63) == 0) {
+        unsigned long long *o = odsd_tl_buf + ((size_t)blockIdx.x * WAVES + (threadIdx.x >> 6)) * 8;
+        for (int k = 0; k < 8; ++k) o[k] = tl[k];
+    }
+#endif
 }
 
 // Shapes the fused kernel is built for; the caller has checked them with odsd_fused_supported().
