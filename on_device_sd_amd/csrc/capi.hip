@@ -64,7 +64,11 @@ static int moe_forward_impl(const odsd_moe_shape *s, const void *x, const void *
                             float *out_f32, void *out_act, int32_t *out_idx, float *out_w,
                             int32_t *out_counts, int32_t *out_offsets, int32_t *out_perm,
                             const double *row_sumsq_in, double *row_sumsq_out,
-                            void *workspace, size_t workspace_bytes, void *stream) {
+                            void *workspace, size_t workspace_bytes, void *stream,
+                            bool prepared = false, const void *next_norm_w = nullptr) {
+    // prepared: the previous block's combine has already applied this block's RMSNorm and left the
+    // normalised rows and their fp16 copy in this workspace; next_norm_w: this block's combine does
+    // the same for the block after it
     if (!s) return ODSD_ERR_NULL;
     const size_t need = odsd_moe_workspace_bytes(s);
     if (need == 0) return ODSD_ERR_SHAPE;
@@ -87,14 +91,16 @@ static int moe_forward_impl(const odsd_moe_shape *s, const void *x, const void *
     // RMSNorm: with the row statistics at hand (left by the previous block's combine) the router
     // kernel normalises on the fly; otherwise the stand-alone kernel runs first
     const void *xin = x;
-    const bool fold = norm_weight && row_sumsq_in;
+    const bool fold = norm_weight && row_sumsq_in && !prepared;
     if (row_sumsq_out && !out_act) return ODSD_ERR_NULL;
-    if (norm_weight && !fold) {
+    if (prepared) {
+        xin = ws + l.xn;
+    } else if (norm_weight && !fold) {
         const int rc = odsd_rmsnorm(x, norm_weight, s->act_dtype, s->T, s->H, eps, ws + l.xn, stream);
         if (rc != ODSD_OK) return rc;
         xin = ws + l.xn;
     }
-    int rc = odsd_launch_router(s, xin, gate_w, idx, w, nullptr, x16, ws + l.router,
+    int rc = odsd_launch_router(s, xin, gate_w, idx, w, nullptr, prepared ? nullptr : x16, ws + l.router,
                                 l.xn - l.router, st, fold ? row_sumsq_in : nullptr, norm_weight, eps,
                                 nullptr, nullptr);
     if (rc != ODSD_OK) return rc;
@@ -107,9 +113,12 @@ static int moe_forward_impl(const odsd_moe_shape *s, const void *x, const void *
         rc = odsd_launch_dispatch(s, idx, counts, offsets, perm, inv, slot_token, st);
         if (rc != ODSD_OK) return rc;
     }
+    // (the combine runs after this block's last reader of xn and x16, so it may overwrite them in place)
+    const OdsdNextNorm nn{next_norm_w, eps, ws + l.xn, x16};
     return odsd_launch_experts(s, x16, table, idx, w, counts, offsets, perm, slot_token,
                                add_residual ? x : nullptr, out_f32, out_act, ws + l.experts,
-                               l.total - l.experts, st, row_sumsq_out, dispatch_inside ? &inside : nullptr);
+                               l.total - l.experts, st, row_sumsq_out, dispatch_inside ? &inside : nullptr,
+                               next_norm_w ? &nn : nullptr);
 }
 
 extern "C" int odsd_moe_forward(const odsd_moe_shape *s, const void *x, const void *norm_weight, float eps,
@@ -210,11 +219,23 @@ static int moe_stack_impl(const odsd_moe_shape *s, int32_t n_layers, const void 
     auto in_of = [&](int l) -> const void * { return l == 0 ? x : hbuf[(l - 1) & 1]; };
     auto out_of = [&](int l) -> void * { return l == n_layers - 1 ? out : hbuf[l & 1]; };
 
+    // Between two blocks the combine of the first applies the RMSNorm of the second (it owns whole
+    // rows and has the row statistic): the second block's router then reads normalised rows and its
+    // expert kernel the fp16 copy, instead of every router workgroup normalising its columns again.  Rows longer than the combine keeps in registers fall back to handing over
+    // the row statistic (the router kernel normalises on the fly).  Same bits either way.
+    const bool hand_rows = odsd_combine_norm_supported(s);
     for (int l = 0; l < n_layers; ++l) {
         begin_layer(l);
-        const int rc = moe_forward_impl(s, in_of(l), norm_w[l], eps, gate_w[l], tables[l], 1, nullptr, out_of(l),
-                                        nullptr, nullptr, nullptr, nullptr, nullptr, l > 0 ? rowss[(l - 1) & 1] : nullptr,
-                                        l + 1 < n_layers ? rowss[l & 1] : nullptr, mws, ml.total, stream);
+        const bool last = l + 1 == n_layers;
+        int rc;
+        if (hand_rows)
+            rc = moe_forward_impl(s, in_of(l), norm_w[l], eps, gate_w[l], tables[l], 1, nullptr, out_of(l),
+                                  nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, mws, ml.total, stream,
+                                  l > 0, last ? nullptr : norm_w[l + 1]);
+        else
+            rc = moe_forward_impl(s, in_of(l), norm_w[l], eps, gate_w[l], tables[l], 1, nullptr, out_of(l),
+                                  nullptr, nullptr, nullptr, nullptr, nullptr, l > 0 ? rowss[(l - 1) & 1] : nullptr,
+                                  last ? nullptr : rowss[l & 1], mws, ml.total, stream);
         end_layer(l);
         if (rc != ODSD_OK) return rc;
     }

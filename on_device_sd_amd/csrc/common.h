@@ -124,6 +124,13 @@ static inline size_t odsd_round_up(size_t v, size_t a) { return (v + a - 1) / a 
 struct OdsdDispatchOut {
     int32_t *counts, *offsets, *perm, *inv, *slot_token;
 };
+// What the combine of a block leaves for the block after it when it is told that block's RMSNorm
+// (calls that run a stack of blocks): the normalised rows in the activation dtype and their fp16 copy.
+struct OdsdNextNorm {
+    const void *norm_w;
+    float eps;
+    void *xn, *x16;
+};
 // router (+ dispatch when `disp` is given)
 int odsd_launch_router(const odsd_moe_shape *s, const void *x, const void *gate_w, int32_t *idx,
                        float *w, int64_t *idx64, void *x16, void *ws, size_t ws_bytes,
@@ -139,5 +146,6 @@ int odsd_launch_experts(const odsd_moe_shape *s, const void *x16, const uint64_t
                         const int32_t *offsets, const int32_t *perm, const int32_t *slot_token,
                         const void *residual, float *out_f32, void *out_act, void *ws,
                         size_t ws_bytes, hipStream_t st, double *row_ss,
-                        const OdsdDispatchOut *dispatch_out = nullptr);
+                        const OdsdDispatchOut *dispatch_out = nullptr, const OdsdNextNorm *next_norm = nullptr);
+int odsd_combine_norm_supported(const odsd_moe_shape *s);
 int odsd_experts_dispatch_inside(const odsd_moe_shape *s);

@@ -447,25 +447,12 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void w4_gemm_kernel(const GemmPara
 // kernel's time consists of at K = 8.
 // YH: 0 = y holds fp32 partial sums of KS slices; 1 = complete sums as fp16; 2 = KS fp16 slices (the
 // batched form, KB > 0, takes exactly two)
-template <typename XT, int YH, bool STATS, int KB>
-__global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ y, const int32_t *__restrict__ idx,
-                                                      const float *__restrict__ w,
-                                                      const int32_t *__restrict__ perm,
-                                                      const uint64_t *__restrict__ table,
-                                                      const XT *__restrict__ residual,
-                                                      float *__restrict__ out_f32, XT *__restrict__ out_act,
-                                                      double *__restrict__ row_ss,
-                                                      int T, int H, int K, int E, int KS, int P, int nchunk) {
-    // One workgroup per (token, 1024-column chunk).  STATS: it also leaves the sum of squares of
-    // what it stored in out_act, row_ss[t][chunk] -- the statistic the next block's RMSNorm
-    // starts from (chunk sums are added in ascending order by whoever consumes them).
-    // (token and chunk share the x dimension of the grid: the y dimension ends at 65535)
-    const int t = blockIdx.x / nchunk;
-    const int chunk = blockIdx.x - t * nchunk;
-    double ss = 0.0;
-    {
-        const int c = (chunk * 256 + threadIdx.x) * 4;
-        if (c < H) {
+// Gather-sum of one token's columns c .. c+3: sum over k of w[t,k] * (sum over slices of y[slice][slot(t,k)]).
+template <int YH, int KB>
+__device__ __forceinline__ float4_t combine_gather(const float *__restrict__ y, const int32_t *__restrict__ idx,
+                                                   const float *__restrict__ w, const int32_t *__restrict__ perm,
+                                                   const uint64_t *__restrict__ table, const int t, const int c,
+                                                   const int H, const int K, const int E, const int KS, const int P) {
         float4_t acc = {0.f, 0.f, 0.f, 0.f};
         if (KB > 0) {
             for (int k0 = 0; k0 < K; k0 += KB) {
@@ -550,23 +537,54 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
             acc.w = fmaf(wk, v.w, acc.w);
         }
         }
-        const size_t o = (size_t)t * H + c;
-        float res[4] = {0.f, 0.f, 0.f, 0.f};
-        if (residual) {
+        return acc;
+}
+
+// What a token's 4 columns become once the sum is there: residual add and the roundings of the
+// reference (out_act = cast(residual + cast(moe))), stores, and the values as stored in out_act.
+template <typename XT>
+__device__ __forceinline__ void combine_finish(const float4_t acc, const XT *__restrict__ residual,
+                                               float *__restrict__ out_f32, XT *__restrict__ out_act,
+                                               const size_t o, float (&stored)[4]) {
+    float res[4] = {0.f, 0.f, 0.f, 0.f};
+    if (residual) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) res[i] = ActIO<XT>::load(residual, o + i);
-        }
-        const float a[4] = {acc.x, acc.y, acc.z, acc.w};
-        if (out_f32) *(float4_t *)(out_f32 + o) = float4_t{a[0] + res[0], a[1] + res[1], a[2] + res[2], a[3] + res[3]};
-        if (out_act) {
+        for (int i = 0; i < 4; ++i) res[i] = ActIO<XT>::load(residual, o + i);
+    }
+    const float a[4] = {acc.x, acc.y, acc.z, acc.w};
+    if (out_f32) *(float4_t *)(out_f32 + o) = float4_t{a[0] + res[0], a[1] + res[1], a[2] + res[2], a[3] + res[3]};
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const float m = ActIO<XT>::round(a[i]);
-                const float stored = ActIO<XT>::round(residual ? __fadd_rn(res[i], m) : m);
-                ActIO<XT>::store(out_act, o + i, stored);
-                if (STATS) ss += (double)stored * (double)stored;
-            }
-        }
+    for (int i = 0; i < 4; ++i) {
+        const float m = ActIO<XT>::round(a[i]);
+        stored[i] = ActIO<XT>::round(residual ? __fadd_rn(res[i], m) : m);
+        if (out_act) ActIO<XT>::store(out_act, o + i, stored[i]);
+    }
+}
+
+template <typename XT, int YH, bool STATS, int KB>
+__global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ y, const int32_t *__restrict__ idx,
+                                                      const float *__restrict__ w,
+                                                      const int32_t *__restrict__ perm,
+                                                      const uint64_t *__restrict__ table,
+                                                      const XT *__restrict__ residual,
+                                                      float *__restrict__ out_f32, XT *__restrict__ out_act,
+                                                      double *__restrict__ row_ss,
+                                                      int T, int H, int K, int E, int KS, int P, int nchunk) {
+    // One workgroup per (token, 1024-column chunk).  STATS: it also leaves the sum of squares of
+    // what it stored in out_act, row_ss[t][chunk] -- the statistic the next block's RMSNorm
+    // starts from (chunk sums are added in ascending order by whoever consumes them).
+    // (token and chunk share the x dimension of the grid: the y dimension ends at 65535)
+    const int t = blockIdx.x / nchunk;
+    const int chunk = blockIdx.x - t * nchunk;
+    double ss = 0.0;
+    const int c = (chunk * 256 + threadIdx.x) * 4;
+    if (c < H) {
+        const float4_t acc = combine_gather<YH, KB>(y, idx, w, perm, table, t, c, H, K, E, KS, P);
+        float stored[4];
+        combine_finish<XT>(acc, residual, out_f32, out_act, (size_t)t * H + c, stored);
+        if (STATS) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) ss += (double)stored[i] * (double)stored[i];
         }
     }
     if (STATS) {
@@ -575,6 +593,59 @@ __global__ __launch_bounds__(256) void combine_kernel(const float *__restrict__ 
         if (lane_id() == 0) red[threadIdx.x >> 6] = ss;
         __syncthreads();
         if (threadIdx.x == 0) row_ss[(size_t)t * nchunk + chunk] = (red[0] + red[1]) + (red[2] + red[3]);
+    }
+}
+
+// The combine of a block whose successor is known (a stack of blocks): one workgroup per token owns
+// the whole row -- 256 threads per 1024-column chunk, each chunk handled exactly as combine_kernel
+// handles it, so the row statistic has the same bits -- and once the statistic is complete it also
+// applies the next block's RMSNorm (demo/src/layers/layernorm.py:21-27, the arithmetic of
+// rmsnorm_kernel and of the router kernel's fold) and leaves what that block starts from: xn, the
+// normalised row in the activation dtype (the next router's input), and x16, its fp16 copy (the
+// expert kernels' operand).  Otherwise every workgroup of the next router kernel that touches the
+// row normalises its columns again (8.2 against 6.0 us per layer at T = 256, H = 2048, E = 128).
+template <typename XT, int YH, int KB>
+__global__ __launch_bounds__(1024) void combine_norm_kernel(const float *__restrict__ y, const int32_t *__restrict__ idx,
+                                                            const float *__restrict__ w,
+                                                            const int32_t *__restrict__ perm,
+                                                            const uint64_t *__restrict__ table,
+                                                            const XT *__restrict__ residual, XT *__restrict__ out_act,
+                                                            int T, int H, int K, int E, int KS, int P,
+                                                            const XT *__restrict__ next_w, double eps,
+                                                            XT *__restrict__ xn_out, half_t *__restrict__ x16_out) {
+    __shared__ double red[16];
+    const int t = blockIdx.x;
+    const int nchunk = (H + 1023) / 1024;              // = blockDim.x / 256
+    const int c = (int)threadIdx.x * 4;                // chunk threadIdx.x / 256, its thread threadIdx.x % 256
+    const bool in = c < H;
+    const size_t o = (size_t)t * H + c;
+    float st[4] = {0.f, 0.f, 0.f, 0.f};
+    float nw[4] = {0.f, 0.f, 0.f, 0.f};
+    double ss = 0.0;
+    if (in) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) nw[i] = ActIO<XT>::load(next_w, c + i);
+        const float4_t acc = combine_gather<YH, KB>(y, idx, w, perm, table, t, c, H, K, E, KS, P);
+        combine_finish<XT>(acc, residual, nullptr, out_act, o, st);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ss += (double)st[i] * (double)st[i];
+    }
+    ss = wave_sum(ss);
+    if (lane_id() == 0) red[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    double tot = 0.0;
+    for (int n = 0; n < nchunk; ++n) tot += (red[4 * n] + red[4 * n + 1]) + (red[4 * n + 2] + red[4 * n + 3]);
+    const double rstd = 1.0 / sqrt(tot / (double)H + eps);
+    if (in) {
+        half4_t h;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float xn = ActIO<XT>::round((float)((double)st[i] * rstd));
+            const float xo = ActIO<XT>::round(__fmul_rn(xn, nw[i]));
+            ActIO<XT>::store(xn_out, o + i, xo);
+            h[i] = f32_to_f16_sat(xo);
+        }
+        *(half4_t *)(x16_out + o) = h;
     }
 }
 
@@ -836,12 +907,16 @@ extern "C" int odsd_w4_down(const odsd_moe_shape *s, const void *h_f16, const ui
     return ODSD_OK;
 }
 
+// the whole-row combine is one workgroup per token, 256 threads per 1024 columns
+int odsd_combine_norm_supported(const odsd_moe_shape *s) { return s && s->H <= 4096 && s->H % 4 == 0; }
+
 // combine: y partials + routing weights (+ residual) -> out (+ per-row sum of squares of out_act)
 // y_slices > 0: y holds that many fp16 partial-sum slices [slice][P][H] (the one-launch expert kernel);
 // 0: the layout of the two-launch plan
 static int launch_combine(const odsd_moe_shape *s, const void *y_, const int32_t *idx, const float *w,
                           const int32_t *perm, const uint64_t *table, const void *residual,
-                          float *out_f32, void *out_act, double *row_ss, hipStream_t st, int y_slices = 0) {
+                          float *out_f32, void *out_act, double *row_ss, hipStream_t st, int y_slices = 0,
+                          const OdsdNextNorm *nn = nullptr) {
     const int rc = experts_args_ok(s);
     if (rc != ODSD_OK) return rc;
     if (s->T == 0) return ODSD_OK;
@@ -858,6 +933,12 @@ static int launch_combine(const odsd_moe_shape *s, const void *y_, const int32_t
     const dim3 grid((unsigned)(nchunk * s->T));
     // rows of 4 pairs fetched together (8: no faster): complete sums, or two fp16 slices
     const bool batched = (pl.KS == 1 || (pl.y_f16 && pl.KS == 2)) && s->K % 4 == 0;
+    if (nn) {
+        // the whole-row form: the next block's normalised input instead of the row statistic
+        if (!odsd_combine_norm_supported(s)) return ODSD_ERR_UNSUPPORTED;
+        if (!out_act || out_f32 || row_ss || !nn->norm_w || !nn->xn || !nn->x16) return ODSD_ERR_NULL;
+        if (!odsd_aligned16(nn->x16) || !odsd_aligned16(nn->xn)) return ODSD_ERR_ALIGN;
+    }
 #define COMBINE_GO(XT, YH, ST)                                                                          \
     do {                                                                                                \
         if (batched)                                                                                    \
@@ -869,9 +950,18 @@ static int launch_combine(const odsd_moe_shape *s, const void *y_, const int32_t
                         table, (const XT *)residual, out_f32, (XT *)out_act, row_ss, s->T, s->H, s->K,  \
                         s->E, pl.KS, P, nchunk);                                                        \
     } while (0)
+#define COMBINE_NORM_N(XT, YH, KB)                                                                      \
+    ODSD_LAUNCH(ODSD_KERNEL_COMBINE, (combine_norm_kernel<XT, YH, KB>), dim3((unsigned)s->T), 256 * nchunk, st, y, idx, w, \
+                perm, table, (const XT *)residual, (XT *)out_act, s->T, s->H, s->K, s->E, pl.KS, P,     \
+                (const XT *)nn->norm_w, (double)nn->eps, (XT *)nn->xn, (half_t *)nn->x16)
 #define COMBINE_Y(XT, ST)                                    \
     do {                                                     \
-        if (pl.y_f16 && pl.KS >= 2) COMBINE_GO(XT, 2, ST);   \
+        if (nn) {                                            \
+            if (pl.y_f16 && pl.KS >= 2) { if (batched) COMBINE_NORM_N(XT, 2, 4); else COMBINE_NORM_N(XT, 2, 0); } \
+            else if (pl.y_f16) { if (batched) COMBINE_NORM_N(XT, 1, 4); else COMBINE_NORM_N(XT, 1, 0); }          \
+            else { if (batched) COMBINE_NORM_N(XT, 0, 4); else COMBINE_NORM_N(XT, 0, 0); }                        \
+        }                                                    \
+        else if (pl.y_f16 && pl.KS >= 2) COMBINE_GO(XT, 2, ST);   \
         else if (pl.y_f16) COMBINE_GO(XT, 1, ST);            \
         else COMBINE_GO(XT, 0, ST);                          \
     } while (0)
@@ -883,6 +973,7 @@ static int launch_combine(const odsd_moe_shape *s, const void *y_, const int32_t
         else COMBINE_Y(float, false);
     }
 #undef COMBINE_Y
+#undef COMBINE_NORM_N
 #undef COMBINE_GO
     ODSD_CHECK_LAUNCH();
     return ODSD_OK;
@@ -898,7 +989,7 @@ int odsd_launch_experts(const odsd_moe_shape *s, const void *x16, const uint64_t
                         const float *w, const int32_t *counts, const int32_t *offsets, const int32_t *perm,
                         const int32_t *slot_token, const void *residual, float *out_f32, void *out_act,
                         void *ws, size_t ws_bytes, hipStream_t st, double *row_ss,
-                        const OdsdDispatchOut *dispatch_out) {
+                        const OdsdDispatchOut *dispatch_out, const OdsdNextNorm *nn) {
     int rc = experts_check(s);
     if (rc != ODSD_OK) return rc;
     if (s->T == 0) return ODSD_OK;
@@ -927,13 +1018,13 @@ int odsd_launch_experts(const odsd_moe_shape *s, const void *x16, const uint64_t
         }
         odsd_launch_experts_fused(fp, s->E, st);
         ODSD_CHECK_LAUNCH();
-        return launch_combine(s, y, idx, w, perm, table, residual, out_f32, out_act, row_ss, st, pl.S);
+        return launch_combine(s, y, idx, w, perm, table, residual, out_f32, out_act, row_ss, st, pl.S, nn);
     }
     rc = launch_gate_up(s, x16, table, counts, offsets, slot_token, h16, st, idx, dispatch_out);
     if (rc != ODSD_OK) return rc;
     rc = odsd_w4_down(s, h16, table, counts, offsets, y, st);
     if (rc != ODSD_OK) return rc;
-    return launch_combine(s, y, idx, w, perm, table, residual, out_f32, out_act, row_ss, st);
+    return launch_combine(s, y, idx, w, perm, table, residual, out_f32, out_act, row_ss, st, 0, nn);
 }
 
 // 1: a whole-block call may skip the dispatch kernel for this shape (the expert kernel scans the
@@ -950,5 +1041,6 @@ extern "C" int odsd_experts_w4(const odsd_moe_shape *s, const void *x_f16, const
                                const void *residual, float *out_f32, void *out_act, void *workspace,
                                size_t workspace_bytes, void *stream) {
     return odsd_launch_experts(s, x_f16, table, idx, w, counts, offsets, perm, slot_token, residual,
-                               out_f32, out_act, workspace, workspace_bytes, (hipStream_t)stream, nullptr);
+                               out_f32, out_act, workspace, workspace_bytes, (hipStream_t)stream, nullptr,
+                               nullptr, nullptr);
 }

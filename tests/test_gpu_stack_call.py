@@ -1,8 +1,8 @@
 """odsd_moe_stack_forward: L blocks in one call (Qwen3DecoderLayer.forward looped over the layers,
 demo/src/layers/decoder_layer.py:126-140, MoE half).  The blocks run the kernels of odsd_moe_forward,
-every block after the first with its RMSNorm folded into the router kernel through the row statistic
-that the previous block's combine leaves -- so the result must equal, bit for bit, the same layers run
-as L whole-block calls; stacks of growing length give the hidden state after every layer, which is
+every block after the first with its RMSNorm applied by the previous block's combine (rows up to 4096
+columns) or folded into the router kernel through the row statistic that combine leaves (longer rows)
+-- either way the result must equal, bit for bit, the same layers run as L whole-block calls; stacks of growing length give the hidden state after every layer, which is
 checked against the oracle teacher-forced.  Router weights with copied and nearly copied rows put exact
 ties and near-ties into the top-k."""
 import numpy as np
@@ -102,16 +102,12 @@ def test_stack_call_layer_by_layer_against_the_oracle(dev, layer, T, ties):
         st.forward_layers(x0.to(dev))
 
 
-def test_stack_call_small_shape_and_arguments(dev):
-    """Another shape (no renormalisation, small experts, the two-launch expert plan), and the call's
-    argument checks."""
-    import ctypes as C
+def _small_stack(dev, T, Hs, Es, Ks, Is, L, dtype, renorm=False, seed=1):
     import on_device_sd_amd as odsd
-    from on_device_sd_amd import _lib
-    T, Hs, Es, Ks, Is, L = 40, 512, 8, 2, 256, 3
-    g = torch.Generator().manual_seed(1)
+    g = torch.Generator().manual_seed(seed)
     cfg = odsd.MoEConfig(hidden_size=Hs, num_hidden_layers=L, num_experts=Es, num_experts_per_token=Ks,
-                         moe_intermediate_size=Is, norm_topk_prob=False)
+                         moe_intermediate_size=Is, norm_topk_prob=renorm,
+                         torch_dtype="float32" if dtype == torch.float32 else "bfloat16")
     banks = []
     for l in range(L):
         bank = odsd.W4ExpertBank(Es, Hs, Is, dev)
@@ -119,10 +115,42 @@ def test_stack_call_small_shape_and_arguments(dev):
             bank.load_expert(e, torch.randn(Is, Hs, generator=g) * 0.02, torch.randn(Is, Hs, generator=g) * 0.02,
                              torch.randn(Hs, Is, generator=g) * 0.02)
         banks.append(bank)
-    gates = [(torch.randn(Es, Hs, generator=g) * 0.02).to(torch.bfloat16) for _ in range(L)]
-    norms = [(1 + 0.1 * torch.randn(Hs, generator=g)).to(torch.bfloat16) for _ in range(L)]
-    x0 = torch.randn(T, Hs, generator=g).to(torch.bfloat16).to(dev)
-    st = odsd.MoEOnlyStack(cfg, gates, norms, banks, T)
+    gates = [(torch.randn(Es, Hs, generator=g) * 0.02).to(dtype) for _ in range(L)]
+    norms = [(1 + 0.1 * torch.randn(Hs, generator=g)).to(dtype) for _ in range(L)]
+    x0 = torch.randn(T, Hs, generator=g).to(dtype).to(dev)
+    return odsd.MoEOnlyStack(cfg, gates, norms, banks, T), x0
+
+
+# rows of one, two (the second partly filled), three and four 1024-column chunks for the whole-row
+# combine, a row shorter than a wavefront's share, fp32 activations, and rows beyond 4096 columns
+# (the row statistic is handed over instead)
+@pytest.mark.parametrize("T,Hs,Es,Ks,Is,dtype", [
+    (40, 512, 8, 2, 256, torch.bfloat16), (24, 4096, 8, 2, 256, torch.bfloat16), (33, 384, 8, 2, 128, torch.float32),
+    (16, 1280, 16, 4, 256, torch.bfloat16), (20, 3072, 8, 2, 128, torch.float32), (9, 128, 4, 1, 128, torch.bfloat16),
+    (8, 5120, 8, 2, 128, torch.bfloat16)])
+def test_stack_call_equals_layer_calls_on_other_shapes(dev, T, Hs, Es, Ks, Is, dtype):
+    print("stack call, shape", T, Hs, Es, Ks, Is, dtype, flush=True)
+    st, x0 = _small_stack(dev, T, Hs, Es, Ks, Is, 3, dtype, renorm=Ks > 1, seed=T)
+    a = st.forward(x0).clone()
+    b = st.forward_layers(x0).clone()
+    torch.cuda.synchronize()
+    assert torch.isfinite(a.float()).all() and torch.equal(a, b)
+    # third way: every layer with the stand-alone RMSNorm kernel in front (no hand-over of any kind)
+    h = [x0.clone(), torch.empty_like(x0)]
+    for l in range(st.L):
+        st.plan.run(h[l & 1], st.gate[l], st.tables[l], st.norm[l], st.config.rms_norm_eps, add_residual=True,
+                    out_act=h[(l + 1) & 1])
+    torch.cuda.synchronize()
+    assert torch.equal(a, h[st.L & 1])
+
+
+def test_stack_call_small_shape_and_arguments(dev):
+    """Another shape (no renormalisation, small experts, the two-launch expert plan), and the call's
+    argument checks."""
+    import ctypes as C
+    from on_device_sd_amd import _lib
+    T, Hs, Es, Ks, Is, L = 40, 512, 8, 2, 256, 3
+    st, x0 = _small_stack(dev, T, Hs, Es, Ks, Is, L, torch.bfloat16)
     a = st.forward(x0).clone()
     b = st.forward_layers(x0).clone()
     assert torch.isfinite(a.float()).all() and torch.equal(a, b)
