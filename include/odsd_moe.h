@@ -227,8 +227,9 @@ int odsd_moe_forward(const odsd_moe_shape *s, const void *x, const void *norm_we
  *   norm_w, gate_w, tables: HOST arrays of n_layers device pointers -- per layer the RMSNorm weight
  *   [H], the router weight [E,H] (both act_dtype) and the expert table (as for odsd_moe_forward)
  * Every layer has the shape *s.  Results are those of n_layers odsd_moe_forward calls with
- * norm_weight and add_residual set, bit for bit (the same kernels; every block after the first takes
- * its RMSNorm statistic from the previous block's combine). */
+ * norm_weight and add_residual set, bit for bit (between two blocks the combine of the first owns
+ * whole rows and applies the RMSNorm of the second; with H > 4096 it hands over the row statistic
+ * and the second block's router kernel normalises on the fly -- the same bits either way). */
 size_t odsd_moe_stack_workspace_bytes(const odsd_moe_shape *s);
 int    odsd_moe_stack_forward(const odsd_moe_shape *s, int32_t n_layers, const void *x,
                               const void *const *norm_w, const void *const *gate_w,
