@@ -19,6 +19,7 @@ from typing import Dict, List, Optional, Sequence
 import torch
 
 from . import _lib
+from .ops import _stream
 
 
 def store_kvcache(key: torch.Tensor, value: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
@@ -51,7 +52,7 @@ def store_kvcache(key: torch.Tensor, value: torch.Tensor, k_cache: torch.Tensor,
                                  k_cache.data_ptr(), v_cache.data_ptr(), slot_mapping.contiguous().data_ptr(),
                                  None if src_index is None else src_index.data_ptr(), N, n, D,
                                  key.element_size(), k_cache.numel() // D,
-                                 torch.cuda.current_stream().cuda_stream), "odsd_kv_store")
+                                 _stream()), "odsd_kv_store")
 
 
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, context: Dict[str, torch.Tensor],
@@ -100,7 +101,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                                         lens.data_ptr(), None if q_lens_dev is None else q_lens_dev.data_ptr(), n_seqs,
                                         mq, num_heads, num_kv_heads, head_dim, block_size,
                                         tables.shape[1], k_cache.numel() // D, scale, dt, out.data_ptr(),
-                                        ws.data_ptr(), nbytes, torch.cuda.current_stream().cuda_stream),
+                                        ws.data_ptr(), nbytes, _stream()),
                "odsd_paged_attention")
     return out
 
@@ -139,7 +140,7 @@ def varlen_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqle
     _lib.check(lib.odsd_varlen_attention(q.data_ptr(), k.data_ptr(), v.data_ptr(), cq.data_ptr(), ck.data_ptr(), n_seqs,
                                          max_seqlen_q, max_seqlen_k, num_heads, num_kv_heads, head_dim, scale, dt,
                                          out.data_ptr(), ws.data_ptr(), nbytes,
-                                         torch.cuda.current_stream().cuda_stream), "odsd_varlen_attention")
+                                         _stream()), "odsd_varlen_attention")
     return out
 
 
