@@ -11,6 +11,9 @@
 #include "common.h"
 
 #define DISPATCH_MAX_WAVES 16
+#ifndef DISPATCH_V4_MIN_PAIRS
+#define DISPATCH_V4_MIN_PAIRS 8193
+#endif
 
 // ITERS > 0: a wavefront's segment is at most 64 * ITERS pairs long and the ids are kept in
 // registers between the two passes; ITERS == 0: any length, the ids are read twice.
@@ -96,6 +99,103 @@ __global__ void dispatch_kernel(const int32_t *__restrict__ idx, int P, int K, i
     }
 }
 
+// Long pair lists (P a multiple of 4): the same scheme with four consecutive ids per lane and load.
+// A wavefront's segment is CH chunks of 256 pairs, all fetched by CH 16-byte loads before the first
+// is looked at.  A lane counts its own matches (0..4), three ballots (one per bit of that count) give
+// the matches in lower lanes and in the chunk, and inside a lane the ids are in pair order -- so the
+// slots are those of the one-id-per-lane form.  (At P = 32768, E = 128 the workgroups read 16 MB of
+// ids from L2 between them: 32 four-byte loads per lane took 14 us.)
+template <int CH>
+__global__ __launch_bounds__(1024) void dispatch_v4_kernel(const int32_t *__restrict__ idx, int P, int K, int E,
+                                                           int32_t *__restrict__ counts,
+                                                           int32_t *__restrict__ offsets,
+                                                           int32_t *__restrict__ perm, int32_t *__restrict__ inv,
+                                                           int32_t *__restrict__ slot_token, uint32_t magic) {
+    __shared__ int s_eq[DISPATCH_MAX_WAVES];
+    __shared__ int s_lt[DISPATCH_MAX_WAVES];
+    typedef int int4_t __attribute__((ext_vector_type(4)));
+    const int e = blockIdx.x;
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int nwaves = blockDim.x >> 6;
+    const int p_begin = wave * (CH * 256);
+    // (the kernel is bound by its instruction count -- 16 wavefronts on one CU per expert, P * E
+    // comparisons in all -- so the first pass only adds up per lane and reduces once per wavefront,
+    // and the match masks it builds are what the second pass works from)
+    int4_t v[CH];
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+        const int p = p_begin + i * 256 + lane * 4;
+        v[i] = p < P ? *(const int4_t *)(idx + p) : int4_t{-1, -1, -1, -1};     // P % 4 == 0: all four or none
+    }
+    uint32_t match[CH];        // bit j: id j of the lane's four belongs to this expert
+    int l_eq = 0, l_lt = 0;
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+        match[i] = (v[i][0] == e ? 1u : 0u) | (v[i][1] == e ? 2u : 0u) | (v[i][2] == e ? 4u : 0u) |
+                   (v[i][3] == e ? 8u : 0u);
+        l_eq += __popc(match[i]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) l_lt += (uint32_t)v[i][j] < (uint32_t)e;     // negative ids compare as huge
+    }
+    const int c_eq = (int)wave_sum((float)l_eq), c_lt = (int)wave_sum((float)l_lt);   // <= 64 * 4 * CH: exact
+    if (lane == 0) { s_eq[wave] = c_eq; s_lt[wave] = c_lt; }
+    __syncthreads();
+    int base = 0, total_eq = 0, total_lt = 0;
+    for (int i = 0; i < nwaves; ++i) {
+        if (i < wave) base += s_eq[i];
+        total_eq += s_eq[i];
+        total_lt += s_lt[i];
+    }
+    if (threadIdx.x == 0) {
+        counts[e] = total_eq;
+        offsets[e] = total_lt;
+        if (e == E - 1) offsets[E] = total_lt + total_eq;
+    }
+    int run = total_lt + base;
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+        const int p = p_begin + i * 256 + lane * 4;
+        const int me = __popc(match[i]);
+        int below = 0, chunk = 0;
+#pragma unroll
+        for (int bit = 0; bit < 3; ++bit) {
+            const uint64_t m = __ballot(me & (1 << bit));
+            below += mask_rank(m) << bit;
+            chunk += __popcll(m) << bit;
+        }
+        int slot = run + below;
+        // Most lanes hold no pair of this expert and few hold two: instead of four predicated rounds
+        // (one per position), the lanes with matches left take their next one, for as many rounds as
+        // the fullest lane needs.
+        uint32_t left = match[i];
+        while (__any(left != 0)) {
+            if (left) {
+                const int j = __builtin_ctz(left);
+                left &= left - 1;
+                const int pj = p + j;
+                perm[pj] = slot;
+                inv[slot] = pj;
+                // pj / K by a multiplication when the host could prove it exact (magic != 0)
+                slot_token[slot] = magic ? (int)__umulhi((uint32_t)pj, magic) : pj / K;
+                ++slot;
+            }
+        }
+        if (e == 0 && p < P) {     // expert 0's workgroup also marks pairs whose id no expert will claim
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (v[i][j] < 0 || v[i][j] >= E) perm[p + j] = -1;
+        }
+        run += chunk;
+    }
+    if (e == E - 1) {
+        for (int s = total_lt + total_eq + (int)threadIdx.x; s < P; s += (int)blockDim.x) {
+            inv[s] = -1;
+            slot_token[s] = -1;
+        }
+    }
+}
+
 int odsd_launch_dispatch(const odsd_moe_shape *s, const int32_t *idx, int32_t *counts, int32_t *offsets,
                          int32_t *perm, int32_t *inv, int32_t *slot_token, hipStream_t st) {
     if (!s) return ODSD_ERR_NULL;
@@ -112,6 +212,24 @@ int odsd_launch_dispatch(const odsd_moe_shape *s, const int32_t *idx, int32_t *c
 #define DISPATCH_GO(IT)                                                                            \
     ODSD_LAUNCH(ODSD_KERNEL_DISPATCH, dispatch_kernel<IT>, s->E, threads, st, idx, P, s->K, s->E, counts, \
                 offsets, perm, inv, slot_token)
+    // four ids per lane and load: wavefronts of CH chunks of 256 pairs, up to 16 of them
+    if (P >= DISPATCH_V4_MIN_PAIRS && P % 4 == 0 && odsd_aligned16(idx) && P <= 16 * 8 * 256) {
+        const int ch = P <= 4096 ? 1 : (P <= 8192 ? 2 : (P <= 16384 ? 4 : 8));
+        const int nw = (P + ch * 256 - 1) / (ch * 256);
+        // floor(p / K) == mulhi(p, floor(2^32 / K) + 1) for every p with p * K < 2^32
+        const uint32_t magic = (uint64_t)P * (uint64_t)s->K < (1ull << 32) && s->K > 1
+                                   ? (uint32_t)((1ull << 32) / (uint32_t)s->K) + 1u : 0u;
+#define DISPATCH_V4(CHV)                                                                                   \
+    ODSD_LAUNCH(ODSD_KERNEL_DISPATCH, dispatch_v4_kernel<CHV>, s->E, 64 * nw, st, idx, P, s->K, s->E, counts, \
+                offsets, perm, inv, slot_token, magic)
+        if (ch == 1) DISPATCH_V4(1);
+        else if (ch == 2) DISPATCH_V4(2);
+        else if (ch == 4) DISPATCH_V4(4);
+        else DISPATCH_V4(8);
+#undef DISPATCH_V4
+        ODSD_CHECK_LAUNCH();
+        return ODSD_OK;
+    }
     if (iters <= 2) DISPATCH_GO(2);
     else if (iters <= 4) DISPATCH_GO(4);
     else if (iters <= 8) DISPATCH_GO(8);

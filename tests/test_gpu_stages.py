@@ -148,7 +148,10 @@ def test_route_dispatch_one_call(dev, T, H, E, K, renorm, dtype):
 
 
 @pytest.mark.parametrize("T,K,E", [(32, 2, 8), (5, 2, 8), (160, 2, 8), (64, 8, 128), (256, 8, 128),
-                                   (4096, 8, 128), (1, 1, 1), (700, 3, 40)])
+                                   (4096, 8, 128), (1, 1, 1), (700, 3, 40),
+                                   # long pair lists (four ids per lane and load): 2.4, 2.9, 4.9 and 8 chunks
+                                   # of 4096 pairs, the last chunks partly filled
+                                   (2500, 4, 64), (1500, 8, 16), (2511, 8, 128), (10001, 1, 7)])
 def test_dispatch_bit_exact(dev, T, K, E):
     print("dispatch", T, K, E, flush=True)
     rng = np.random.default_rng(T + K + E)
@@ -163,6 +166,21 @@ def test_dispatch_bit_exact(dev, T, K, E):
     assert np.array_equal(d.perm.cpu().numpy(), perm)
     assert np.array_equal(d.inv.cpu().numpy(), inv)
     assert np.array_equal(d.slot_token.cpu().numpy(), inv // K)
+
+
+def test_dispatch_long_list_with_ids_nobody_claims(dev):
+    print("dispatch long list, out-of-range ids", flush=True)
+    rng = np.random.default_rng(5)
+    T, K, E = 3000, 4, 32
+    idx = rng.integers(0, E, size=(T, K)).astype(np.int32)
+    idx[rng.random((T, K)) < 0.05] = -1
+    idx[rng.random((T, K)) < 0.05] = E + 3
+    d = _ops().dispatch(torch.from_numpy(idx).to(dev), E)
+    c, o, perm, inv = orc.dispatch(idx, E)
+    assert np.array_equal(d.counts.cpu().numpy(), c)
+    assert np.array_equal(d.offsets.cpu().numpy(), o)
+    assert np.array_equal(d.perm.cpu().numpy(), perm)
+    assert np.array_equal(d.inv.cpu().numpy(), inv)
 
 
 def test_dispatch_duplicates_and_out_of_range(dev):
