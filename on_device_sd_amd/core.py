@@ -79,8 +79,9 @@ class RoutingResult:
     (for example on a hand-built RoutingResult).  ``x_f16`` is the fp16 copy of the routed
     hidden states that the router kernel writes anyway, tagged with the identity of the tensor
     it was made from; forward_moe uses it when it is handed that same, unmodified tensor
-    (unmodified as far as torch's version counter tells: a caller that overwrites the routed
-    tensor in place through something other than torch must clear ``x_f16``).
+    (unmodified as far as torch's version counter tells; this package's own calls move that
+    counter for every buffer they overwrite, so only a caller that rewrites the routed tensor
+    through a foreign kernel must clear ``x_f16``).
     """
     layer_idx: int
     topk_indices: torch.Tensor

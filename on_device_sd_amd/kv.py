@@ -19,7 +19,7 @@ from typing import Dict, List, Optional, Sequence
 import torch
 
 from . import _lib
-from .ops import _stream
+from .ops import _stream, _wrote
 
 
 def store_kvcache(key: torch.Tensor, value: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
@@ -53,6 +53,7 @@ def store_kvcache(key: torch.Tensor, value: torch.Tensor, k_cache: torch.Tensor,
                                  None if src_index is None else src_index.data_ptr(), N, n, D,
                                  key.element_size(), k_cache.numel() // D,
                                  _stream()), "odsd_kv_store")
+    _wrote(k_cache, v_cache)
 
 
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, context: Dict[str, torch.Tensor],

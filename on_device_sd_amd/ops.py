@@ -39,6 +39,19 @@ def _stream() -> int:
     return torch.cuda.current_stream().cuda_stream
 
 
+def _wrote(*tensors: Optional[torch.Tensor]) -> None:
+    """Tell torch that the library has overwritten these tensors in place.  A kernel launched through
+    ctypes is invisible to torch's modification counter, and that counter is what the runner keys its
+    reuse of the router's fp16 copy on: buffers that live across calls (a plan's outputs, a buffer the
+    caller handed in) must not look unchanged after a call has rewritten them."""
+    for t in tensors:
+        if t is not None:
+            _increment_version(t)
+
+
+_increment_version = getattr(torch.autograd.graph, "increment_version", None) or (lambda t: t.add_(0))
+
+
 def _require_cuda(*tensors: torch.Tensor) -> None:
     for t in tensors:
         if t is not None and not t.is_cuda:
@@ -363,6 +376,7 @@ class MoeForwardPlan:
             _ptr(self.w), _ptr(self.counts), _ptr(self.offsets), _ptr(self.perm),
             _ptr(row_sumsq_in), _ptr(row_sumsq_out), self.ws.data_ptr(),
             self.ws.numel(), _stream()), "odsd_moe_forward")
+        _wrote(self.out_f32, oa)
         return MoeOutputs(self.out_f32, oa, self.idx, self.w, self.counts, self.offsets, self.perm)
 
     def run_events(self, events, x: torch.Tensor, gate_weight: torch.Tensor, table: torch.Tensor,
@@ -381,6 +395,7 @@ class MoeForwardPlan:
             table.data_ptr(), 1 if add_residual else 0, _ptr(self.out_f32), _ptr(oa),
             _ptr(row_sumsq_in), _ptr(row_sumsq_out), self.ws.data_ptr(), self.ws.numel(), _stream(),
             events.array, C.byref(mask)), "odsd_moe_forward_events")
+        _wrote(self.out_f32, oa)
         return mask.value
 
 
@@ -408,6 +423,7 @@ class MoeStackPlan:
         _lib.check(lib.odsd_moe_stack_forward(C.byref(self.shape), self.L, x.data_ptr(), self._norm, self._gate,
                                               self._tables, self.eps, self.out.data_ptr(), self.ws.data_ptr(),
                                               self.ws.numel(), _stream()), "odsd_moe_stack_forward")
+        _wrote(self.out)
         return self.out
 
     def run_events(self, events, x: torch.Tensor):
@@ -420,6 +436,7 @@ class MoeStackPlan:
             C.byref(self.shape), self.L, x.data_ptr(), self._norm, self._gate, self._tables, self.eps,
             self.out.data_ptr(), self.ws.data_ptr(), self.ws.numel(), _stream(), events.array, masks),
             "odsd_moe_stack_forward_events")
+        _wrote(self.out)
         return list(masks)
 
 
@@ -473,3 +490,4 @@ class ExpertStages:
         _lib.check(lib.odsd_combine(C.byref(self.shape), self.y.data_ptr(), idx.data_ptr(), w.data_ptr(),
                                     disp.perm.data_ptr(), table.data_ptr(), _ptr(residual), _ptr(out_f32),
                                     _ptr(out_act), _stream()), "odsd_combine")
+        _wrote(out_f32, out_act)

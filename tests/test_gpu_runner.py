@@ -219,6 +219,22 @@ def test_router_fp16_copy_is_reused_only_for_the_routed_tensor(runner, dev):
     # the routed tensor modified in place after routing: its version counter has moved on
     hidden.mul_(0.5)
     check_output(run(hidden), orc.forward_moe(hidden.cpu(), hidden.cpu(), idx, sc, runner.oracle_experts[0]))
+    # the routed tensor overwritten in place by one of the library's own calls (a plan writing its
+    # output into the caller's buffer): torch sees no kernel, the library says so itself
+    from on_device_sd_amd import ops
+    cfg = runner.config
+    res2 = runner.route_experts(0, hidden)
+    idx2, sc2 = res2.topk_indices.cpu().numpy(), res2.topk_scores.cpu().numpy()
+    plan = ops.MoeForwardPlan(7, H, cfg.num_experts, cfg.num_experts_per_token, cfg.moe_intermediate_size,
+                              cfg.norm_topk_prob, hidden.dtype, dev, want_f32=False)
+    src = _hidden(dev, 7, H, seed=8)
+    before = hidden.clone()
+    plan.run(src, runner.gate_weights[0], runner.banks[0].table(), add_residual=True, out_act=hidden)
+    torch.cuda.synchronize()
+    assert not torch.equal(hidden, before)
+    placement = odsd.ExpertPlacement(gpu_expert_params=params, cpu_expert_params={}, routing_result=res2)
+    check_output(runner.forward_moe(0, _attn(hidden), placement),
+                 orc.forward_moe(hidden.cpu(), hidden.cpu(), idx2, sc2, runner.oracle_experts[0]))
 
 
 def test_placement_tables_are_cached_by_parameter_identity(runner, dev):
