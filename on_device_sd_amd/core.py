@@ -81,7 +81,8 @@ class RoutingResult:
     it was made from; forward_moe uses it when it is handed that same, unmodified tensor
     (unmodified as far as torch's version counter tells; this package's own calls move that
     counter for every buffer they overwrite, so only a caller that rewrites the routed tensor
-    through a foreign kernel must clear ``x_f16``).
+    through a foreign kernel must clear ``x_f16``; tensors made under ``torch.inference_mode()``
+    have no counter, and for them any in-place rewrite between the two calls needs that).
     """
     layer_idx: int
     topk_indices: torch.Tensor

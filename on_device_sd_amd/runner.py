@@ -212,8 +212,11 @@ class W4MoERunner:
 
 def _tensor_tag(t: torch.Tensor) -> tuple:
     """Identity of a tensor's contents as far as the host can tell: storage address, shape,
-    dtype and the in-place modification counter."""
-    return (t.data_ptr(), tuple(t.shape), t.dtype, t._version)
+    dtype and the in-place modification counter.  Tensors made under ``torch.inference_mode()``
+    (the reference's executor steps run under it, cb_executor.py:302) carry no counter: for
+    them the tag is address, shape and dtype, and an in-place overwrite between route_experts
+    and forward_moe goes unseen -- the engine's steps hand the routed tensor on untouched."""
+    return (t.data_ptr(), tuple(t.shape), t.dtype, -1 if t.is_inference() else t._version)
 
 
 # -- stateless forms ---------------------------------------------------------------------------

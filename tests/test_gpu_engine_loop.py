@@ -265,3 +265,13 @@ def test_prefill_then_decode_steps_through_the_context_builders(dev):
                               None, KVH, BS, HD ** -0.5)
     err = (out.float().cpu() - ref).abs()
     assert err.max().item() <= 2e-2 and err.mean().item() <= 2e-3
+
+
+def test_steps_under_inference_mode(dev, tmp_path):
+    """The reference's executor runs its steps under torch.inference_mode() (cb_executor.py:302,
+    :349, :405): tensors made there have no version counter and may not be touched by autograd's
+    book-keeping.  The engine-loop, draft-step and prefill / decode flows above, once more inside it."""
+    with torch.inference_mode():
+        test_engine_loop_over_three_layers(dev, tmp_path)
+        test_draft_step_with_substitution_from_the_builder(dev, tmp_path)
+        test_prefill_then_decode_steps_through_the_context_builders(dev)

@@ -237,6 +237,38 @@ def test_router_fp16_copy_is_reused_only_for_the_routed_tensor(runner, dev):
                  orc.forward_moe(hidden.cpu(), hidden.cpu(), idx2, sc2, runner.oracle_experts[0]))
 
 
+def test_engine_calls_under_inference_mode(runner, dev):
+    """The reference's executor steps run under torch.inference_mode() (cb_executor.py:302): the
+    tensors carry no version counter there, and the two calls must work all the same."""
+    import on_device_sd_amd as odsd
+    with torch.inference_mode():
+        hidden = _hidden(dev, 9, H, seed=12) * 1.0          # an inference tensor
+        assert hidden.is_inference()
+        res = runner.route_experts(0, hidden)
+        placement = odsd.build_prefill_placement(res, _NoCache(), _BankLoader(runner.banks[0]))
+        out = runner.forward_moe(0, _attn(hidden), placement)
+        layer = runner.forward_layer(0, hidden) if runner.norm_weights is not None else None
+    idx, sc = res.topk_indices.cpu().numpy(), res.topk_scores.cpu().numpy()
+    check_output(out, orc.forward_moe(hidden.cpu(), hidden.cpu(), idx, sc, runner.oracle_experts[0]))
+    assert layer is None or torch.isfinite(layer.hidden_states.float()).all()
+
+
+class _NoCache:
+    def is_cached(self, expert_id):
+        return False
+
+
+class _BankLoader:
+    def __init__(self, bank):
+        self.bank = bank
+
+    def is_shared_expert(self, expert_id):
+        return False
+
+    def get_expert_params(self, expert_id, device=None):
+        return self.bank.expert_params(expert_id.expert_idx)
+
+
 def test_placement_tables_are_cached_by_parameter_identity(runner, dev):
     import on_device_sd_amd as odsd
     bank = runner.banks[0]

@@ -163,3 +163,10 @@ def test_verify_step_equals_successive_decode_steps(dev):
         out_d = odsd.paged_attention(qj, kc, vc, ctx_d, KV, bs)
         diff = (out_d.float() - out_v[:, j].float()).abs().max().item()
         assert diff <= 4e-3, (j, diff)      # different key slicing and rounding points, same sums
+
+
+def test_verify_step_under_inference_mode(dev):
+    """The whole verify step (norms, KV store, paged attention, routing, placement, experts) inside
+    torch.inference_mode(), as the reference's executor runs it (cb_executor.py:349)."""
+    with torch.inference_mode():
+        test_verify_step_through_two_layers(dev)
