@@ -64,6 +64,27 @@ def test_static_scratch_matches_workspace_call(dev):
         assert int(ref["counts"].sum()) == T * K and torch.isfinite(ref["out_f32"]).all()
 
 
+def test_static_scratch_call_at_the_one_launch_shape(dev):
+    """The Qwen3-30B-A3B layer shape (one-launch expert kernel with the dispatch inside, 29 MiB of
+    workspace) through the static array, then a smaller call over what it left behind."""
+    from on_device_sd_amd import _lib
+    lib = _lib.load()
+    H, E, K, I = 2048, 128, 8, 768
+    gate, bank, x, norm = _layer(dev, 256, H, E, K, I, 31)
+    for T in (256, 136):
+        print("no-alloc entry point, one-launch shape: T", T, flush=True)
+        shape = _lib.MoeShape(T, H, E, K, I, 1, _lib.DT_BF16, 0)
+        assert lib.odsd_experts_one_launch(C.byref(shape)) == 1
+        assert lib.odsd_moe_workspace_bytes(C.byref(shape)) <= _lib.STATIC_SCRATCH_BYTES
+        xt = x[:T].contiguous()
+        got = _run(lib, True, shape, xt, norm, gate, bank.table(), dev)
+        ref = _run(lib, False, shape, xt, norm, gate, bank.table(), dev)
+        for name in ref:
+            assert torch.equal(got[name].view(torch.uint8), ref[name].view(torch.uint8)), \
+                f"T={T}: {name} differs between the static-scratch call and the workspace call"
+        assert int(ref["counts"].sum()) == T * K and torch.isfinite(ref["out_f32"]).all()
+
+
 def test_static_scratch_call_under_graph_capture(dev):
     """The use the entry point is offered for: after odsd_moe_static_init() the call is captured into
     a HIP graph (nothing may allocate or query the runtime there) and replayed several times, with
