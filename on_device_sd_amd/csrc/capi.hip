@@ -100,19 +100,17 @@ static int moe_forward_impl(const odsd_moe_shape *s, const void *x, const void *
         if (rc != ODSD_OK) return rc;
         xin = ws + l.xn;
     }
-    int rc = odsd_launch_router(s, xin, gate_w, idx, w, nullptr, prepared ? nullptr : x16, ws + l.router,
-                                l.xn - l.router, st, fold ? row_sumsq_in : nullptr, norm_weight, eps,
-                                nullptr, nullptr);
-    if (rc != ODSD_OK) return rc;
     // shapes served by the one-launch expert kernel need no dispatch kernel: its workgroups scan the
     // expert ids themselves and leave counts / offsets / perm (inv and slot_token are not produced:
-    // nothing after the experts reads them)
+    // nothing after the experts reads them); otherwise the router launch dispatches as well (with few
+    // tokens inside its top-k kernel, else by the dispatch kernel)
     const OdsdDispatchOut inside{counts, offsets, perm, nullptr, nullptr};
+    const OdsdDispatchOut outside{counts, offsets, perm, inv, slot_token};
     const bool dispatch_inside = odsd_experts_dispatch_inside(s) && odsd_aligned16(idx);
-    if (!dispatch_inside) {
-        rc = odsd_launch_dispatch(s, idx, counts, offsets, perm, inv, slot_token, st);
-        if (rc != ODSD_OK) return rc;
-    }
+    int rc = odsd_launch_router(s, xin, gate_w, idx, w, nullptr, prepared ? nullptr : x16, ws + l.router,
+                                l.xn - l.router, st, fold ? row_sumsq_in : nullptr, norm_weight, eps,
+                                nullptr, dispatch_inside ? nullptr : &outside);
+    if (rc != ODSD_OK) return rc;
     // (the combine runs after this block's last reader of xn and x16, so it may overwrite them in place)
     const OdsdNextNorm nn{next_norm_w, eps, ws + l.xn, x16};
     return odsd_launch_experts(s, x16, table, idx, w, counts, offsets, perm, slot_token,

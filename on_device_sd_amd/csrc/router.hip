@@ -208,15 +208,12 @@ __global__ __launch_bounds__(256) void router_partial_kernel(const XT *__restric
 }
 
 // V = logits per lane (experts lane, lane + 64, ...): 1, 2, 4 or 8 for E <= 64, 128, 256, 512
+// the selection for token t by one wavefront; lane k < K returns the k-th winner's expert id
 template <int V>
-__global__ __launch_bounds__(256) void router_topk_kernel(const double *__restrict__ partial, int T, int E,
-                                                          int K, int S, int renorm,
-                                                          int32_t *__restrict__ idx,
-                                                          float *__restrict__ w,
-                                                          int64_t *__restrict__ idx64,
-                                                          double *__restrict__ logits) {
-    const int t = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-    if (t >= T) return;
+__device__ __forceinline__ int topk_token(const double *__restrict__ partial, const int t, int T, int E,
+                                          int K, int S, int renorm, int32_t *__restrict__ idx,
+                                          float *__restrict__ w, int64_t *__restrict__ idx64,
+                                          double *__restrict__ logits) {
     const int lane = lane_id();
 
     double lg[V];
@@ -296,6 +293,59 @@ __global__ __launch_bounds__(256) void router_topk_kernel(const double *__restri
         idx[o] = my_e;
         w[o] = num / den;
         if (idx64) idx64[o] = (int64_t)my_e;
+    }
+    return my_e;
+}
+
+template <int V>
+__global__ __launch_bounds__(256) void router_topk_kernel(const double *__restrict__ partial, int T, int E,
+                                                          int K, int S, int renorm,
+                                                          int32_t *__restrict__ idx,
+                                                          float *__restrict__ w,
+                                                          int64_t *__restrict__ idx64,
+                                                          double *__restrict__ logits) {
+    const int t = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (t >= T) return;
+    topk_token<V>(partial, t, T, E, K, S, renorm, idx, w, idx64, logits);
+}
+
+// Few tokens (T <= 16, P = T * K <= ROUTER_SMALL_PAIRS): one workgroup, one wavefront per token, and
+// behind a barrier the same workgroup sorts the pairs by expert -- the dispatch of dispatch.hip on a
+// list that fits LDS, without its launch (decode and short verify steps: 4 us of a 107 us layer at
+// T = 5).  Thread p owns pair p: its slot is the number of pairs of lower experts plus the number of
+// earlier pairs of its own expert, which is the stable order of the dispatch kernel.
+#define ROUTER_SMALL_PAIRS 128
+template <int V>
+__global__ __launch_bounds__(1024) void router_topk_dispatch_small_kernel(
+    const double *__restrict__ partial, int T, int E, int K, int S, int renorm, int32_t *__restrict__ idx,
+    float *__restrict__ w, int64_t *__restrict__ idx64, double *__restrict__ logits,
+    int32_t *__restrict__ counts, int32_t *__restrict__ offsets, int32_t *__restrict__ perm,
+    int32_t *__restrict__ inv, int32_t *__restrict__ slot_token) {
+    __shared__ int32_t ids[ROUTER_SMALL_PAIRS];
+    const int t = threadIdx.x >> 6, lane = lane_id();
+    if (t < T) {
+        const int my_e = topk_token<V>(partial, t, T, E, K, S, renorm, idx, w, idx64, logits);
+        if (lane < K) ids[t * K + lane] = my_e;
+    }
+    __syncthreads();
+    const int P = T * K;
+    for (int e = threadIdx.x; e < E; e += blockDim.x) {
+        int c = 0, lt = 0;
+        for (int q = 0; q < P; ++q) {
+            c += ids[q] == e;
+            lt += ids[q] < e;
+        }
+        counts[e] = c;
+        offsets[e] = lt;
+        if (e == E - 1) offsets[E] = lt + c;
+    }
+    if ((int)threadIdx.x < P) {
+        const int pq = threadIdx.x, e = ids[pq];
+        int slot = 0;
+        for (int q = 0; q < P; ++q) slot += ids[q] < e || (ids[q] == e && q < pq);
+        perm[pq] = slot;
+        inv[slot] = pq;
+        slot_token[slot] = pq / K;
     }
 }
 
@@ -394,6 +444,19 @@ int odsd_launch_router(const odsd_moe_shape *s, const void *x, const void *gate_
     const int S_out = p.S % 4 == 0 ? p.S / 4 : p.S;
     // one wavefront per token; with few tokens each gets a workgroup of its own (a CU to itself:
     // 4.4 against 4.9 us at T = 256), with many, four share one (8.6 against 9.8 us at T = 4096)
+    if (disp && s->T <= 16 && s->K <= 64 && s->T * s->K <= ROUTER_SMALL_PAIRS) {
+#define TOPK_SMALL_GO(VV)                                                                                      \
+    ODSD_LAUNCH(ODSD_KERNEL_ROUTER_TOPK, router_topk_dispatch_small_kernel<VV>, 1, 64 * s->T, st,               \
+                (const double *)partial, s->T, s->E, s->K, S_out, s->renorm, idx, w, idx64, logits, disp->counts, \
+                disp->offsets, disp->perm, disp->inv, disp->slot_token)
+        if (s->E <= 64) TOPK_SMALL_GO(1);
+        else if (s->E <= 128) TOPK_SMALL_GO(2);
+        else if (s->E <= 256) TOPK_SMALL_GO(4);
+        else TOPK_SMALL_GO(8);
+#undef TOPK_SMALL_GO
+        ODSD_CHECK_LAUNCH();
+        return ODSD_OK;
+    }
     const int tk_waves = s->T <= 512 ? 1 : 4;
 #define TOPK_GO(VV)                                                                                   \
     ODSD_LAUNCH(ODSD_KERNEL_ROUTER_TOPK, router_topk_kernel<VV>, (s->T + tk_waves - 1) / tk_waves, 64 * tk_waves, st, \
