@@ -312,8 +312,8 @@ __global__ __launch_bounds__(256) void router_topk_kernel(const double *__restri
 // Few tokens (T <= 16, P = T * K <= ROUTER_SMALL_PAIRS): one workgroup, one wavefront per token, and
 // behind a barrier the same workgroup sorts the pairs by expert -- the dispatch of dispatch.hip on a
 // list that fits LDS, without its launch (decode and short verify steps: 4 us of a 107 us layer at
-// T = 5).  Thread p owns pair p: its slot is the number of pairs of lower experts plus the number of
-// earlier pairs of its own expert, which is the stable order of the dispatch kernel.
+// T = 5).  A pair's slot is the number of pairs of lower experts plus the number of earlier pairs of
+// its own expert, which is the stable order of the dispatch kernel.
 #define ROUTER_SMALL_PAIRS 128
 template <int V>
 __global__ __launch_bounds__(1024) void router_topk_dispatch_small_kernel(
@@ -328,24 +328,32 @@ __global__ __launch_bounds__(1024) void router_topk_dispatch_small_kernel(
         if (lane < K) ids[t * K + lane] = my_e;
     }
     __syncthreads();
-    const int P = T * K;
-    for (int e = threadIdx.x; e < E; e += blockDim.x) {
-        int c = 0, lt = 0;
-        for (int q = 0; q < P; ++q) {
-            c += ids[q] == e;
-            lt += ids[q] < e;
+    // wavefront w sorts out experts w, w + nw, ...: the pair list sits in two registers per lane (pairs
+    // lane and lane + 64), ballots count the pairs of the expert and of lower experts, and the lanes
+    // that hold a pair of the expert take consecutive slots in pair order
+    const int P = T * K, nw = blockDim.x >> 6;
+    const int id0 = lane < P ? ids[lane] : -1, id1 = lane + 64 < P ? ids[lane + 64] : -1;
+    for (int e = t; e < E; e += nw) {
+        const uint64_t m0 = __ballot(id0 == e), m1 = __ballot(id1 == e);
+        const int c0 = __popcll(m0), c = c0 + __popcll(m1);
+        const int lt = __popcll(__ballot(id0 >= 0 && id0 < e)) + __popcll(__ballot(id1 >= 0 && id1 < e));
+        if (lane == 0) {
+            counts[e] = c;
+            offsets[e] = lt;
+            if (e == E - 1) offsets[E] = lt + c;
         }
-        counts[e] = c;
-        offsets[e] = lt;
-        if (e == E - 1) offsets[E] = lt + c;
-    }
-    if ((int)threadIdx.x < P) {
-        const int pq = threadIdx.x, e = ids[pq];
-        int slot = 0;
-        for (int q = 0; q < P; ++q) slot += ids[q] < e || (ids[q] == e && q < pq);
-        perm[pq] = slot;
-        inv[slot] = pq;
-        slot_token[slot] = pq / K;
+        if (id0 == e) {
+            const int slot = lt + mask_rank(m0);
+            perm[lane] = slot;
+            inv[slot] = lane;
+            slot_token[slot] = lane / K;
+        }
+        if (id1 == e) {
+            const int slot = lt + c0 + mask_rank(m1);
+            perm[lane + 64] = slot;
+            inv[slot] = lane + 64;
+            slot_token[slot] = (lane + 64) / K;
+        }
     }
 }
 
@@ -444,9 +452,14 @@ int odsd_launch_router(const odsd_moe_shape *s, const void *x, const void *gate_
     const int S_out = p.S % 4 == 0 ? p.S / 4 : p.S;
     // one wavefront per token; with few tokens each gets a workgroup of its own (a CU to itself:
     // 4.4 against 4.9 us at T = 256), with many, four share one (8.6 against 9.8 us at T = 4096)
-    if (disp && s->T <= 16 && s->K <= 64 && s->T * s->K <= ROUTER_SMALL_PAIRS) {
+    // (one CU then runs every token's selection: with 2 logits per lane 16 tokens take 10.2 us against
+    // 8.6 for the two kernels, 5 tokens 7.2 against 8.4; with one logit per lane 16 tokens 5.4 against 8.1)
+    const int topk_v = s->E <= 64 ? 1 : (s->E <= 128 ? 2 : (s->E <= 256 ? 4 : 8));
+    if (disp && s->T * topk_v <= 16 && s->K <= 64 && s->T * s->K <= ROUTER_SMALL_PAIRS) {
+        // a wavefront per token, and enough of them that the sort has at most 8 experts each
+        const int small_waves = max(s->T, min(16, (s->E + 7) / 8));
 #define TOPK_SMALL_GO(VV)                                                                                      \
-    ODSD_LAUNCH(ODSD_KERNEL_ROUTER_TOPK, router_topk_dispatch_small_kernel<VV>, 1, 64 * s->T, st,               \
+    ODSD_LAUNCH(ODSD_KERNEL_ROUTER_TOPK, router_topk_dispatch_small_kernel<VV>, 1, 64 * small_waves, st,        \
                 (const double *)partial, s->T, s->E, s->K, S_out, s->renorm, idx, w, idx64, logits, disp->counts, \
                 disp->offsets, disp->perm, disp->inv, disp->slot_token)
         if (s->E <= 64) TOPK_SMALL_GO(1);
