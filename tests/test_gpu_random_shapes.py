@@ -2,6 +2,8 @@
 plan boundary (direct path up to 16 tokens, 32-, 64- and 128-row streaming passes, the tile kernel),
 odd group counts, top-1 to top-8, both activation dtypes, both weight rules, experts without weights
 and substituted experts.  Routing bit-exact, outputs in tolerance, every case twice for determinism."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -30,7 +32,9 @@ def _cases(n, seed):
     return out
 
 
-CASES = _cases(64, 20240607)
+# (more cases or another seed for a longer run: ODSD_RANDOM_SHAPES="count,seed")
+_N, _SEED = (int(v) for v in os.environ.get("ODSD_RANDOM_SHAPES", "64,20240607").split(","))
+CASES = _cases(_N, _SEED)
 
 
 @pytest.mark.parametrize("case", CASES, ids=lambda c: f"{c[0]}-T{c[1]}-H{c[2]}-E{c[3]}-K{c[4]}-I{c[5]}")
