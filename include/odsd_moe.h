@@ -51,8 +51,9 @@ extern "C" {
 /* 110: events / static forms of the whole block, KV store, paged and packed attention added (100: the MoE block)
  * 112: odsd_moe_shape.max_rows (was reserved, 0 keeps the old meaning), odsd_experts_one_launch
  * 113: odsd_moe_static_init
- * 114: odsd_moe_stack_forward, odsd_moe_stack_forward_events */
-#define ODSD_VERSION 114
+ * 114: odsd_moe_stack_forward, odsd_moe_stack_forward_events
+ * 115: odsd_route_dispatch_host_counts */
+#define ODSD_VERSION 115
 
 typedef enum odsd_status {
     ODSD_OK = 0,
@@ -154,6 +155,19 @@ int odsd_route_dispatch(const odsd_moe_shape *s, const void *x, const void *gate
                         int32_t *out_idx, float *out_w, int64_t *out_idx64, void *x_f16,
                         int32_t *counts, int32_t *offsets, int32_t *perm, int32_t *inv,
                         int32_t *slot_token, void *workspace, size_t workspace_bytes, void *stream);
+
+/* The same call with a second copy of the counts written by the kernel itself to counts_host: [E] int64
+ * in pinned host memory that the device can address (hipHostMalloc), entry e = (tag << 32) | counts[e],
+ * one 8-byte store each.  The engine reads the activated set on the host between routing and
+ * execution (qwen3_runner.py:110-112).  A device-to-host copy on the stream in front of the experts
+ * cost 4 to 11 us per layer, an event record 3 to 5; with the tag (a number the caller changes from
+ * call to call) the host can tell from the buffer alone when every entry has arrived, and nothing
+ * but the kernels sits on the stream.  counts_host may be null (then this is odsd_route_dispatch). */
+int odsd_route_dispatch_host_counts(const odsd_moe_shape *s, const void *x, const void *gate_w,
+                                    int32_t *out_idx, float *out_w, int64_t *out_idx64, void *x_f16,
+                                    int32_t *counts, int32_t *offsets, int32_t *perm, int32_t *inv,
+                                    int32_t *slot_token, int64_t *counts_host, uint32_t tag, void *workspace,
+                                    size_t workspace_bytes, void *stream);
 
 /* ---- Dispatch ----------------------------------------------------------------------- */
 /* Stable counting sort of the P pairs by expert id.

@@ -43,6 +43,8 @@ SIGNATURES = {
     "odsd_router_topk": (C.c_int, [_SP, _P, _P, _P, _P, _P, _P, _P, C.c_size_t, _P]),
     "odsd_router_topk_logits": (C.c_int, [_SP, _P, _P, _P, _P, _P, _P, _P, _P, C.c_size_t, _P]),
     "odsd_route_dispatch": (C.c_int, [_SP, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, C.c_size_t, _P]),
+    "odsd_route_dispatch_host_counts": (C.c_int, [_SP, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, C.c_uint32,
+                                                  _P, C.c_size_t, _P]),
     "odsd_convert_act_f16": (C.c_int, [_P, C.c_int32, C.c_int64, _P, _P]),
     "odsd_dispatch": (C.c_int, [_SP, _P, _P, _P, _P, _P, _P, _P]),
     "odsd_experts_workspace_bytes": (C.c_size_t, [_SP]),

@@ -123,6 +123,10 @@ static inline size_t odsd_round_up(size_t v, size_t a) { return (v + a - 1) / a 
 // dispatch arrays a router launch may fill as well (all five or none)
 struct OdsdDispatchOut {
     int32_t *counts, *offsets, *perm, *inv, *slot_token;
+    // optional second copy of counts for the host (memory the device can write), or null: entry e is
+    // (mirror_tag << 32) | counts[e], so a reader that knows the tag can tell when entry e has arrived
+    int64_t *counts_mirror;
+    uint32_t mirror_tag;
 };
 // What the combine of a block leaves for the block after it when it is told that block's RMSNorm
 // (calls that run a stack of blocks): the normalised rows in the activation dtype and their fp16 copy.
@@ -138,7 +142,7 @@ int odsd_launch_router(const odsd_moe_shape *s, const void *x, const void *gate_
                        double *logits = nullptr, const OdsdDispatchOut *disp = nullptr);
 int odsd_launch_dispatch(const odsd_moe_shape *s, const int32_t *idx, int32_t *counts,
                          int32_t *offsets, int32_t *perm, int32_t *inv, int32_t *slot_token,
-                         hipStream_t st);
+                         hipStream_t st, int64_t *counts_mirror = nullptr, uint32_t mirror_tag = 0u);
 // dispatch_out: the dispatch arrays have NOT been filled; the expert kernel dispatches for itself and
 // leaves counts / offsets / perm there (only when odsd_experts_dispatch_inside(s) says it can)
 int odsd_launch_experts(const odsd_moe_shape *s, const void *x16, const uint64_t *table,

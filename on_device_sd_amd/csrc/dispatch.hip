@@ -21,7 +21,8 @@ template <int ITERS>
 __global__ void dispatch_kernel(const int32_t *__restrict__ idx, int P, int K, int E,
                                 int32_t *__restrict__ counts, int32_t *__restrict__ offsets,
                                 int32_t *__restrict__ perm, int32_t *__restrict__ inv,
-                                int32_t *__restrict__ slot_token) {
+                                int32_t *__restrict__ slot_token, int64_t *__restrict__ counts_mirror,
+                                uint32_t mirror_tag) {
     __shared__ int s_eq[DISPATCH_MAX_WAVES];
     __shared__ int s_lt[DISPATCH_MAX_WAVES];
     const int e = blockIdx.x;
@@ -64,6 +65,8 @@ __global__ void dispatch_kernel(const int32_t *__restrict__ idx, int P, int K, i
     }
     if (threadIdx.x == 0) {
         counts[e] = total_eq;
+        // a tagged second copy, e.g. in host memory the device can write: one 8-byte store per expert
+        if (counts_mirror) counts_mirror[e] = (int64_t)(((uint64_t)mirror_tag << 32) | (uint32_t)total_eq);
         offsets[e] = total_lt;
         if (e == E - 1) offsets[E] = total_lt + total_eq;
     }
@@ -110,7 +113,8 @@ __global__ __launch_bounds__(1024) void dispatch_v4_kernel(const int32_t *__rest
                                                            int32_t *__restrict__ counts,
                                                            int32_t *__restrict__ offsets,
                                                            int32_t *__restrict__ perm, int32_t *__restrict__ inv,
-                                                           int32_t *__restrict__ slot_token, uint32_t magic) {
+                                                           int32_t *__restrict__ slot_token, uint32_t magic,
+                                                           int64_t *__restrict__ counts_mirror, uint32_t mirror_tag) {
     __shared__ int s_eq[DISPATCH_MAX_WAVES];
     __shared__ int s_lt[DISPATCH_MAX_WAVES];
     typedef int int4_t __attribute__((ext_vector_type(4)));
@@ -149,6 +153,8 @@ __global__ __launch_bounds__(1024) void dispatch_v4_kernel(const int32_t *__rest
     }
     if (threadIdx.x == 0) {
         counts[e] = total_eq;
+        // a tagged second copy, e.g. in host memory the device can write: one 8-byte store per expert
+        if (counts_mirror) counts_mirror[e] = (int64_t)(((uint64_t)mirror_tag << 32) | (uint32_t)total_eq);
         offsets[e] = total_lt;
         if (e == E - 1) offsets[E] = total_lt + total_eq;
     }
@@ -197,7 +203,8 @@ __global__ __launch_bounds__(1024) void dispatch_v4_kernel(const int32_t *__rest
 }
 
 int odsd_launch_dispatch(const odsd_moe_shape *s, const int32_t *idx, int32_t *counts, int32_t *offsets,
-                         int32_t *perm, int32_t *inv, int32_t *slot_token, hipStream_t st) {
+                         int32_t *perm, int32_t *inv, int32_t *slot_token, hipStream_t st, int64_t *counts_mirror,
+                         uint32_t mirror_tag) {
     if (!s) return ODSD_ERR_NULL;
     if (s->T < 0 || s->E <= 0 || s->K <= 0) return ODSD_ERR_SHAPE;
     if ((int64_t)s->T * s->K > 0x7fffffffLL) return ODSD_ERR_SHAPE;
@@ -211,7 +218,7 @@ int odsd_launch_dispatch(const odsd_moe_shape *s, const int32_t *idx, int32_t *c
     const int iters = (((P + nwaves - 1) / nwaves + 63) & ~63) / 64;   // 64-pair chunks per wavefront
 #define DISPATCH_GO(IT)                                                                            \
     ODSD_LAUNCH(ODSD_KERNEL_DISPATCH, dispatch_kernel<IT>, s->E, threads, st, idx, P, s->K, s->E, counts, \
-                offsets, perm, inv, slot_token)
+                offsets, perm, inv, slot_token, counts_mirror, mirror_tag)
     // four ids per lane and load: wavefronts of CH chunks of 256 pairs, up to 16 of them
     if (P >= DISPATCH_V4_MIN_PAIRS && P % 4 == 0 && odsd_aligned16(idx) && P <= 16 * 8 * 256) {
         const int ch = P <= 4096 ? 1 : (P <= 8192 ? 2 : (P <= 16384 ? 4 : 8));
@@ -221,7 +228,7 @@ int odsd_launch_dispatch(const odsd_moe_shape *s, const int32_t *idx, int32_t *c
                                    ? (uint32_t)((1ull << 32) / (uint32_t)s->K) + 1u : 0u;
 #define DISPATCH_V4(CHV)                                                                                   \
     ODSD_LAUNCH(ODSD_KERNEL_DISPATCH, dispatch_v4_kernel<CHV>, s->E, 64 * nw, st, idx, P, s->K, s->E, counts, \
-                offsets, perm, inv, slot_token, magic)
+                offsets, perm, inv, slot_token, magic, counts_mirror, mirror_tag)
         if (ch == 1) DISPATCH_V4(1);
         else if (ch == 2) DISPATCH_V4(2);
         else if (ch == 4) DISPATCH_V4(4);
@@ -243,5 +250,5 @@ int odsd_launch_dispatch(const odsd_moe_shape *s, const int32_t *idx, int32_t *c
 extern "C" int odsd_dispatch(const odsd_moe_shape *s, const int32_t *idx, int32_t *counts,
                              int32_t *offsets, int32_t *perm, int32_t *inv, int32_t *slot_token,
                              void *stream) {
-    return odsd_launch_dispatch(s, idx, counts, offsets, perm, inv, slot_token, (hipStream_t)stream);
+    return odsd_launch_dispatch(s, idx, counts, offsets, perm, inv, slot_token, (hipStream_t)stream, nullptr, 0u);
 }

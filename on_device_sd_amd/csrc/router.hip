@@ -320,7 +320,8 @@ __global__ __launch_bounds__(1024) void router_topk_dispatch_small_kernel(
     const double *__restrict__ partial, int T, int E, int K, int S, int renorm, int32_t *__restrict__ idx,
     float *__restrict__ w, int64_t *__restrict__ idx64, double *__restrict__ logits,
     int32_t *__restrict__ counts, int32_t *__restrict__ offsets, int32_t *__restrict__ perm,
-    int32_t *__restrict__ inv, int32_t *__restrict__ slot_token) {
+    int32_t *__restrict__ inv, int32_t *__restrict__ slot_token, int64_t *__restrict__ counts_mirror,
+    uint32_t mirror_tag) {
     __shared__ int32_t ids[ROUTER_SMALL_PAIRS];
     const int t = threadIdx.x >> 6, lane = lane_id();
     if (t < T) {
@@ -339,6 +340,7 @@ __global__ __launch_bounds__(1024) void router_topk_dispatch_small_kernel(
         const int lt = __popcll(__ballot(id0 >= 0 && id0 < e)) + __popcll(__ballot(id1 >= 0 && id1 < e));
         if (lane == 0) {
             counts[e] = c;
+            if (counts_mirror) counts_mirror[e] = (int64_t)(((uint64_t)mirror_tag << 32) | (uint32_t)c);
             offsets[e] = lt;
             if (e == E - 1) offsets[E] = lt + c;
         }
@@ -461,7 +463,7 @@ int odsd_launch_router(const odsd_moe_shape *s, const void *x, const void *gate_
 #define TOPK_SMALL_GO(VV)                                                                                      \
     ODSD_LAUNCH(ODSD_KERNEL_ROUTER_TOPK, router_topk_dispatch_small_kernel<VV>, 1, 64 * small_waves, st,        \
                 (const double *)partial, s->T, s->E, s->K, S_out, s->renorm, idx, w, idx64, logits, disp->counts, \
-                disp->offsets, disp->perm, disp->inv, disp->slot_token)
+                disp->offsets, disp->perm, disp->inv, disp->slot_token, disp->counts_mirror, disp->mirror_tag)
         if (s->E <= 64) TOPK_SMALL_GO(1);
         else if (s->E <= 128) TOPK_SMALL_GO(2);
         else if (s->E <= 256) TOPK_SMALL_GO(4);
@@ -480,7 +482,9 @@ int odsd_launch_router(const odsd_moe_shape *s, const void *x, const void *gate_
     else TOPK_GO(8);
 #undef TOPK_GO
     ODSD_CHECK_LAUNCH();
-    if (disp) return odsd_launch_dispatch(s, idx, disp->counts, disp->offsets, disp->perm, disp->inv, disp->slot_token, st);
+    if (disp)
+        return odsd_launch_dispatch(s, idx, disp->counts, disp->offsets, disp->perm, disp->inv, disp->slot_token, st,
+                                    disp->counts_mirror, disp->mirror_tag);
     return ODSD_OK;
 }
 
@@ -496,6 +500,16 @@ extern "C" int odsd_route_dispatch(const odsd_moe_shape *s, const void *x, const
                                    int32_t *counts, int32_t *offsets, int32_t *perm, int32_t *inv,
                                    int32_t *slot_token, void *workspace, size_t workspace_bytes, void *stream) {
     const OdsdDispatchOut d{counts, offsets, perm, inv, slot_token};
+    return odsd_launch_router(s, x, gate_w, out_idx, out_w, out_idx64, x_f16, workspace, workspace_bytes,
+                              (hipStream_t)stream, nullptr, nullptr, 0.0f, nullptr, &d);
+}
+
+extern "C" int odsd_route_dispatch_host_counts(const odsd_moe_shape *s, const void *x, const void *gate_w,
+                                               int32_t *out_idx, float *out_w, int64_t *out_idx64, void *x_f16,
+                                               int32_t *counts, int32_t *offsets, int32_t *perm, int32_t *inv,
+                                               int32_t *slot_token, int64_t *counts_host, uint32_t tag,
+                                               void *workspace, size_t workspace_bytes, void *stream) {
+    const OdsdDispatchOut d{counts, offsets, perm, inv, slot_token, counts_host, tag};
     return odsd_launch_router(s, x, gate_w, out_idx, out_w, out_idx64, x_f16, workspace, workspace_bytes,
                               (hipStream_t)stream, nullptr, nullptr, 0.0f, nullptr, &d);
 }

@@ -236,9 +236,13 @@ def dispatch(idx: torch.Tensor, num_experts: int, idx32_keep: bool = False) -> D
 
 
 def route_dispatch(x: torch.Tensor, gate_weight: torch.Tensor, top_k: int, renorm: bool,
-                   want_f16: bool = True, want_int64: bool = True):
+                   want_f16: bool = True, want_int64: bool = True,
+                   counts_host: Optional[torch.Tensor] = None, counts_tag: int = 0):
     """Router, top-k and dispatch in one library call.
-    Returns (idx int32 [T,K], w float32 [T,K], idx64 or None, x_f16 or None, Dispatch)."""
+    Returns (idx int32 [T,K], w float32 [T,K], idx64 or None, x_f16 or None, Dispatch).
+    ``counts_host``: a pinned int64 [E] host tensor that the dispatch kernel fills as well, entry e =
+    (counts_tag << 32) | counts[e] (the device writes it directly: no copy and no event on the stream;
+    an entry has arrived when its upper half shows the tag)."""
     _require_cuda(x, gate_weight)
     lib = _lib.load()
     if gate_weight.dtype != x.dtype:
@@ -260,19 +264,24 @@ def route_dispatch(x: torch.Tensor, gate_weight: torch.Tensor, top_k: int, renor
     w = torch.empty(T, top_k, dtype=torch.float32, device=dev)
     idx64 = torch.empty(T, top_k, dtype=torch.int64, device=dev) if want_int64 else None
     x16 = torch.empty(T, H, dtype=torch.float16, device=dev) if want_f16 else None
+    if counts_host is not None and not (counts_host.is_pinned() and counts_host.dtype == torch.int64
+                                        and counts_host.is_contiguous() and counts_host.numel() == E):
+        raise ValueError("counts_host must be a pinned, contiguous int64 [E] host tensor")
     if T == 0:
         d.counts.zero_()
         d.offsets.zero_()
+        if counts_host is not None:
+            counts_host.fill_((counts_tag & 0xffffffff) << 32)
         return idx, w, idx64, x16, d
     nbytes = lib.odsd_router_workspace_bytes(C.byref(shape))
     if nbytes == 0:
         raise _lib.OdsdError(f"router: unsupported shape T={T} H={H} E={E} K={top_k}")
     ws = _workspace(nbytes, dev)
-    _lib.check(lib.odsd_route_dispatch(C.byref(shape), x.data_ptr(), gate_weight.data_ptr(), idx.data_ptr(),
-                                       w.data_ptr(), _ptr(idx64), _ptr(x16), d.counts.data_ptr(),
-                                       d.offsets.data_ptr(), d.perm.data_ptr(), d.inv.data_ptr(),
-                                       d.slot_token.data_ptr(), ws.data_ptr(), ws.numel(), _stream()),
-               "odsd_route_dispatch")
+    _lib.check(lib.odsd_route_dispatch_host_counts(
+        C.byref(shape), x.data_ptr(), gate_weight.data_ptr(), idx.data_ptr(), w.data_ptr(), _ptr(idx64), _ptr(x16),
+        d.counts.data_ptr(), d.offsets.data_ptr(), d.perm.data_ptr(), d.inv.data_ptr(), d.slot_token.data_ptr(),
+        _ptr(counts_host), counts_tag & 0xffffffff, ws.data_ptr(), ws.numel(), _stream()),
+        "odsd_route_dispatch_host_counts")
     return idx, w, idx64, x16, d
 
 

@@ -27,7 +27,7 @@ def test_every_declared_symbol_is_exported_and_bound():
 
 def test_version_and_status_strings():
     lib = _lib.load()
-    assert lib.odsd_version() == 114
+    assert lib.odsd_version() == 115
     assert lib.odsd_status_string(0) == b"ok"
     for code in range(1, 9):
         assert len(lib.odsd_status_string(code)) > 3

@@ -124,6 +124,8 @@ def test_router_ties_lower_index_first(dev):
     (3, 384, 5, 3, True, torch.bfloat16),       # odd number of column groups
     (1, 128, 1, 1, False, torch.float32),
     (40, 512, 60, 6, False, torch.bfloat16),
+    (64, 256, 128, 8, True, torch.bfloat16),    # the dispatch kernel, one id per lane
+    (1200, 128, 16, 8, True, torch.bfloat16),   # 9600 pairs: four ids per lane and load
 ])
 def test_route_dispatch_one_call(dev, T, H, E, K, renorm, dtype):
     print("route_dispatch", T, H, E, K, renorm, dtype, flush=True)
@@ -139,6 +141,13 @@ def test_route_dispatch_one_call(dev, T, H, E, K, renorm, dtype):
     assert np.array_equal(d.counts.cpu().numpy(), c) and np.array_equal(d.offsets.cpu().numpy(), o)
     assert np.array_equal(d.perm.cpu().numpy(), perm) and np.array_equal(d.inv.cpu().numpy(), inv)
     assert np.array_equal(d.slot_token.cpu().numpy(), inv // K)
+    # the counts once more in pinned host memory, written by the dispatch kernel itself and tagged
+    host = torch.zeros(E, dtype=torch.int64, pin_memory=True)
+    _ops().route_dispatch(x.to(dev), wg.to(dev), K, renorm, counts_host=host, counts_tag=0x80000007)
+    torch.cuda.synchronize()
+    got = host.numpy().view(np.uint64)
+    assert np.array_equal(got >> np.uint64(32), np.full(E, 0x80000007, np.uint64))
+    assert np.array_equal((got & np.uint64(0xffffffff)).astype(np.int32), c)
     # the separate calls give the same bits
     idx2, w2, _, _ = _ops().router_topk(x.to(dev), wg.to(dev), K, renorm)
     assert torch.equal(idx2, idx) and torch.equal(w2, w)
